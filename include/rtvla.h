@@ -1,0 +1,150 @@
+/* rtvla - C ABI of the MI355X (gfx950) Pi0 / Pi05 single-observation forward pass.
+ *
+ * The reference (Dexmal/realtime-vla) has no native layer: its device code is Triton JIT and its
+ * "operator interface" is the Python object Pi0Inference / Pi05Inference.  This ABI is what a
+ * Python (ctypes) front end with that object's signature binds instead of the Triton kernels.
+ * Every entry point takes plain pointers and sizes, returns an int status (0 = ok, see
+ * rtvla_status) and never throws; device memory is always owned by the caller.
+ *
+ * Life cycle:   rtvla_create -> rtvla_bind (every weight / io buffer) -> rtvla_bind_workspace
+ *            -> rtvla_prepare -> [rtvla_graph_capture] -> rtvla_forward / rtvla_graph_launch ...
+ *            -> rtvla_destroy.
+ * One context = one static shape set (views, prompt length, chunk); single host thread per
+ * context; calls that enqueue work on the same context must not overlap.
+ */
+#ifndef RTVLA_H
+#define RTVLA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct rtvla_ctx rtvla_ctx;
+
+enum rtvla_status {
+    RTVLA_OK = 0,
+    RTVLA_ERR_ARG = 1,        /* null pointer, bad size, unsupported dimension            */
+    RTVLA_ERR_NAME = 2,       /* unknown tensor name                                       */
+    RTVLA_ERR_SIZE = 3,       /* byte size does not match the tensor's shape               */
+    RTVLA_ERR_STATE = 4,      /* call out of order (e.g. forward before prepare)           */
+    RTVLA_ERR_UNBOUND = 5,    /* a required tensor was never bound                         */
+    RTVLA_ERR_DEVICE = 6,     /* HIP runtime error; text in rtvla_last_error               */
+    RTVLA_ERR_LIMIT = 7       /* shape outside the supported range                         */
+};
+
+enum rtvla_model { RTVLA_PI0 = 0, RTVLA_PI05 = 1 };
+
+/* Static shape set of one inference object.
+ * Replaces the constructor arguments and literals of Pi0Inference.__init__
+ * (/root/reference/pi0_infer.py:1239-1243, :1289-1290) and Pi05Inference.__init__
+ * (/root/reference/pi05_infer.py:531-561, :615-616). */
+typedef struct rtvla_dims {
+    int32_t model;           /* rtvla_model                                                          */
+    int32_t num_views;       /* 1..4 camera views of 224x224x3                                        */
+    int32_t prompt_len;      /* Pi0: rows of language_embeds; Pi05: max_prompt_len (allocated rows)   */
+    int32_t chunk_size;      /* action chunk; Pi0 suffix = chunk+1 rows, Pi05 = chunk rows (<= 64)    */
+    int32_t num_steps;       /* Euler flow steps (the reference hard-codes 10)                        */
+    int32_t vision_layers;   /* SigLIP layers (27)                                                    */
+    int32_t llm_layers;      /* Gemma prefix layers == action-expert layers (18)                      */
+} rtvla_dims;
+
+/* Stages of the forward schedule, for per-stage execution (layer taps, profiling).
+ * A whole forward is: VISION_EMBED, VISION_LAYER x vision_layers, PROJECT,
+ * PREFIX_LAYER x llm_layers, SUFFIX_INIT, then per step SUFFIX_STEP_BEGIN,
+ * SUFFIX_LAYER x llm_layers, SUFFIX_STEP_END. */
+enum rtvla_stage {
+    RTVLA_STAGE_VISION_EMBED = 0,   /* pi0_infer.py:348-364 conv2d_embed_n256_1152_res               */
+    RTVLA_STAGE_VISION_LAYER = 1,   /* pi0_infer.py:607-646 one SigLIP layer                         */
+    RTVLA_STAGE_PROJECT = 2,        /* pi0_infer.py:753-775 + :1344 final LN, projector, prompt rows */
+    RTVLA_STAGE_PREFIX_LAYER = 3,   /* pi0_infer.py:851-884 one Gemma prefix layer (KV cache fill)   */
+    RTVLA_STAGE_SUFFIX_INIT = 4,    /* pi0_infer.py:1166-1171 state token (Pi0 only)                 */
+    RTVLA_STAGE_SUFFIX_STEP_BEGIN = 5, /* pi0_infer.py:1173-1185 / pi05_infer.py:420-425             */
+    RTVLA_STAGE_SUFFIX_LAYER = 6,   /* pi0_infer.py:1186-1223 / pi05_infer.py:427-509                */
+    RTVLA_STAGE_SUFFIX_STEP_END = 7 /* pi0_infer.py:1224-1230 / pi05_infer.py:511-523 Euler update   */
+};
+
+/* Library build / ABI version (no reference counterpart). */
+int rtvla_version(void);
+
+/* Create a context for one shape set.  Replaces the tensor allocation block of
+ * Pi0Inference.__init__ (pi0_infer.py:1245-1317) / Pi05Inference.__init__ (pi05_infer.py:563-653):
+ * validates the dimensions and lays out the workspace; allocates no device memory. */
+int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out);
+
+/* Release host state (device memory belongs to the caller). */
+int rtvla_destroy(rtvla_ctx* ctx);
+
+/* Text of the last error on this context (never null). */
+const char* rtvla_last_error(const rtvla_ctx* ctx);
+
+/* Number of tensors the context knows by name, and their description: name, element size,
+ * rank and shape (up to 4 dims), whether it is a weight (1) or an io buffer (0), and whether
+ * it must be bound before rtvla_prepare.  Names and shapes are exactly the keys of
+ * `self.weights` / `self.buffers` in the reference (pi0_infer.py:1245-1317,
+ * pi05_infer.py:563-653) for the tensors that cross the boundary. */
+int rtvla_tensor_count(const rtvla_ctx* ctx);
+int rtvla_tensor_info(const rtvla_ctx* ctx, int index, const char** name, int32_t* elem_bytes,
+                      int32_t* rank, int64_t shape[4], int32_t* is_weight, int32_t* required);
+
+/* Bind a caller-owned device tensor by its reference name; `bytes` must equal the tensor's size.
+ * Replaces `self.weights[k].copy_(v)` (pi0_infer.py:1337-1338): the library reads the caller's
+ * tensor in place.  Unknown name -> RTVLA_ERR_NAME (the reference raises KeyError). */
+int rtvla_bind(rtvla_ctx* ctx, const char* name, void* device_ptr, size_t bytes);
+
+/* Bytes of scratch the context needs (re-tiled weights, activations, KV cache), and binding of a
+ * caller-owned, 256-byte aligned device allocation of at least that size. */
+size_t rtvla_workspace_bytes(const rtvla_ctx* ctx);
+int rtvla_bind_workspace(rtvla_ctx* ctx, void* device_ptr, size_t bytes);
+
+/* Location of a named internal activation inside the workspace, for taps and for the
+ * `buffers` views of the Python object: byte offset, rows, cols, leading dimension (elements),
+ * element size.  Names follow the reference's buffer keys where one exists (vision_x, encoder_x,
+ * encoder_K, decoder_x, ...); encoder_Vt is the transposed V cache. */
+int rtvla_buffer_count(const rtvla_ctx* ctx);
+int rtvla_buffer_info(const rtvla_ctx* ctx, int index, const char** name, size_t* offset,
+                      int64_t* rows, int64_t* cols, int64_t* ld, int32_t* elem_bytes);
+
+/* One-time device work after all weights are bound: re-tile weights into MFMA fragment order,
+ * clear the workspace, Pi05: scale the output projection by -1/num_steps and compute the
+ * time-conditioning style vectors (pi05_infer.py:669-722).  Enqueued on `hip_stream` (a
+ * hipStream_t passed as void*); the caller synchronises. */
+int rtvla_prepare(rtvla_ctx* ctx, void* hip_stream);
+
+/* Enqueue one whole forward (pi0_model pi0_infer.py:1232-1236 / pi05_model pi05_infer.py:525-528)
+ * on the stream: no allocation, no synchronisation, no host read - capturable.  Inputs are read
+ * from the bound io buffers; the result is left in `diffusion_noise`. */
+int rtvla_forward(rtvla_ctx* ctx, void* hip_stream);
+
+/* Enqueue a single stage (see rtvla_stage); `layer` and `step` are ignored where meaningless. */
+int rtvla_forward_stage(rtvla_ctx* ctx, int stage, int layer, int step, void* hip_stream);
+
+/* Capture rtvla_forward into a HIP graph held by the context / replay it on a stream.
+ * Replaces record_infer_graph and infer_graph.replay() (pi0_infer.py:1347-1354, :1360). */
+int rtvla_graph_capture(rtvla_ctx* ctx, void* hip_stream);
+int rtvla_graph_launch(rtvla_ctx* ctx, void* hip_stream);
+
+/* Number of kernel launches one forward enqueues (graph nodes). */
+int rtvla_launch_count(const rtvla_ctx* ctx);
+
+/* Measurement helper (no reference counterpart): run `stage` `iters` times back to back on the
+ * stream between two HIP events recorded on that same stream and return the mean milliseconds
+ * per run.  Synchronises the stream. */
+int rtvla_time_stage(rtvla_ctx* ctx, int stage, int layer, int step, int iters, void* hip_stream, float* mean_ms);
+
+/* Measurement helper: time `iters` graph replays (or eager forwards when no graph is captured)
+ * individually with HIP events on the stream; writes per-iteration milliseconds to ms_out[iters]. */
+int rtvla_time_forward(rtvla_ctx* ctx, int iters, void* hip_stream, float* ms_out);
+
+/* Unit-level entry points used by the parity tests: run one kernel family on caller tensors.
+ * `w_tiled` comes from rtvla_pretile.  (No reference counterpart; the reference's per-kernel
+ * wrappers, e.g. pi0_infer.py:396-419, :727-733, take torch tensors.) */
+size_t rtvla_pretile_elems(int K, int N);
+int rtvla_pretile(const void* w, int K, int N, void* w_tiled, void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RTVLA_H */

@@ -1,0 +1,77 @@
+"""Shared host logic of Pi0Inference / Pi05Inference: tensor ownership (PyTorch-ROCm), binding
+to the C ABI, RoPE tables, graph capture.  PyTorch is used only to own device memory and for
+the input staging copies; every kernel of the forward lives in librtvla.so."""
+import torch
+
+import rtvla_capi as capi
+
+_DTYPES = {2: torch.bfloat16, 4: torch.int32}
+
+
+def rope_table(start, count, device):
+    """Rows [cos_0, sin_0, cos_1, sin_1, ...] in bf16 for positions start..start+count-1
+    (/root/reference/pi0_infer.py:1319-1335)."""
+    position_ids = torch.arange(start, start + count, device=device)
+    inv_freq = 1.0 / (10000 ** (torch.arange(0, 256, 2, dtype=torch.float32, device=device) / 256))
+    phase = inv_freq[None, :] * position_ids[:, None]
+    cos = torch.cos(phase).to(torch.bfloat16)
+    sin = torch.sin(phase).to(torch.bfloat16)
+    return torch.cat([cos[:, :, None], sin[:, :, None]], 2).view(-1, 256)
+
+
+class Engine:
+    def __init__(self, model, checkpoint, num_views, prompt_len, chunk_size, num_steps=10, skip_keys=()):
+        if not torch.cuda.is_available():
+            raise RuntimeError("realtime-vla_amd needs a ROCm GPU (MI355X / gfx950); there is no CPU path")
+        self.device = torch.device("cuda", torch.cuda.current_device())
+        vision_layers, llm_layers = 27, 18
+        if "vision_attn_qkv_w" in checkpoint:
+            vision_layers = int(checkpoint["vision_attn_qkv_w"].shape[0])
+        if "encoder_attn_qkv_w" in checkpoint:
+            llm_layers = int(checkpoint["encoder_attn_qkv_w"].shape[0])
+        self.ctx = capi.Context(model, num_views, prompt_len, chunk_size, num_steps, vision_layers, llm_layers)
+        self.weights, self.buffers = {}, {}
+        for name, elem, shape, is_weight, _ in self.ctx.tensors():
+            # zero-initialised so that a weight the checkpoint omits (the reference leaves it
+            # uninitialised, benchmark.py:9-11) can never inject NaN/Inf
+            t = torch.zeros(*shape, dtype=_DTYPES[elem], device=self.device)
+            (self.weights if is_weight else self.buffers)[name] = t
+        for k, v in checkpoint.items():
+            if k in skip_keys:
+                continue
+            if not torch.is_tensor(v):
+                v = torch.as_tensor(v)
+            self.weights[k].copy_(v)               # KeyError on an unknown key, RuntimeError on a shape mismatch
+        for name, t in list(self.weights.items()) + list(self.buffers.items()):
+            self.ctx.bind(name, t.data_ptr(), t.numel() * t.element_size())
+        nbytes = self.ctx.workspace_bytes()
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        self.ctx.bind_workspace(self.workspace.data_ptr(), nbytes)
+        # views of the library's internal activations, under the reference's buffer names where one exists
+        for name, off, rows, cols, ld, elem in self.ctx.buffers():
+            if name.startswith("t_"):
+                continue
+            flat = self.workspace[off:off + rows * ld * elem].view(torch.bfloat16 if elem == 2 else torch.float32)
+            self.buffers.setdefault(name, flat.view(rows, ld)[:, :cols])
+        self.stream = torch.cuda.current_stream(self.device)
+
+    def prepare(self):
+        self.ctx.prepare(self.stream.cuda_stream)
+        torch.cuda.synchronize(self.device)
+
+    def capture(self):
+        """One eager forward, then capture into a HIP graph on a side stream
+        (/root/reference/pi0_infer.py:1347-1354)."""
+        side = torch.cuda.Stream(self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        self.ctx.graph_capture(side.cuda_stream)
+        side.synchronize()
+
+    def replay(self):
+        self.ctx.graph_launch(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def run_stage(self, stage, layer=0, step=0):
+        self.ctx.forward_stage(stage, layer, step, torch.cuda.current_stream(self.device).cuda_stream)
+
+    def run_eager(self):
+        self.ctx.forward(torch.cuda.current_stream(self.device).cuda_stream)

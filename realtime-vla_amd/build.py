@@ -1,0 +1,50 @@
+"""Build librtvla.so (gfx950) in-tree with hipcc: python build.py [--force]."""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "librtvla.so")
+SOURCES = ["gemm.hip", "skinny.hip", "attention.hip", "misc.hip", "rtvla.hip"]
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-unused-value",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _hipcc():
+    for p in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if p and (os.path.sep not in p or os.path.exists(p)):
+            return p
+    return "hipcc"
+
+
+def _compile(src):
+    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+    cmd = [_hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "warnings generated" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s" % (src, err))
+    return obj, err
+
+
+def build(force=True, verbose=False):
+    """Compile every HIP source for gfx950 and link the shared library."""
+    if not force and os.path.exists(LIB):
+        return LIB
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4)) as ex:
+        results = list(ex.map(_compile, SOURCES))
+    if verbose:
+        for _, err in results:
+            if err.strip():
+                print(err)
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + [o for o, _ in results]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force=True, verbose="-v" in sys.argv))

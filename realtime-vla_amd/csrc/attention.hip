@@ -1,0 +1,267 @@
+// Softmax attention on MFMA, flash style (online softmax, logits never leave registers).
+//
+//  * mqa_kernel    - Gemma multi-query attention, 8 query heads sharing one 256-wide K/V head: the
+//                    prefix pass (/root/reference/pi0_infer.py:819-824, pi05_infer.py:335-360) and
+//                    the action-expert suffix pass with its masks (pi0_infer.py:1041-1120,
+//                    pi05_infer.py:382-478).  Query rows are token*8 + head, so the whole thing is
+//                    a [rows x 256] x [keys x 256]^T problem against one shared K and V.
+//  * vision_kernel - SigLIP attention, 16 heads x 72 per view, 256 keys (pi0_infer.py:588-596).
+//
+// Both compute the transposed logits S^T = K Q^T so that each lane holds 16 keys of ONE query row:
+// the softmax statistics are per-lane scalars and the probabilities are already in the register
+// layout of the MFMA B operand for O^T = V^T P^T, provided V is read with the matching key
+// permutation.  V is therefore kept transposed in memory ([d][key]) by the producing GEMM.
+#include "kernels.h"
+
+namespace {
+
+constexpr float NEG_BIG = -1.0e30f;
+
+RTVLA_DEVICE bf16x8 cat44(bf16x4 lo, bf16x4 hi) {
+    bf16x8 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { v[j] = lo[j]; v[4 + j] = hi[j]; }
+    return v;
+}
+
+template <int WAVES, int MQ>
+__global__ __launch_bounds__(WAVES * 64)
+void mqa_kernel(AttnP p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    f32x4* obuf = (f32x4*)smem_raw;                                   // [WAVES][16][64]
+    float* ms = (float*)(smem_raw + (size_t)WAVES * 16 * 64 * 16);    // [WAVES][MQ][16]
+    float* ls = ms + WAVES * MQ * 16;                                 // [WAVES][MQ][16]
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int g = lane >> 4, r = lane & 15;
+    const int m0 = blockIdx.x * (16 * MQ);
+
+    int vl = p.prefix_alloc;
+    if (p.valid_len) vl = max(0, min(*p.valid_len, p.prefix_alloc));
+
+    bf16x8 qf[MQ][8];
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+        const int row = min(m0 + mq * 16 + r, p.rows - 1);
+        const bf16_t* qp = p.q + (size_t)row * p.ldq + 8 * g;
+#pragma unroll
+        for (int kd = 0; kd < 8; ++kd) qf[mq][kd] = *(const bf16x8*)(qp + kd * 32);
+    }
+    f32x4 o[MQ][16];
+    float mrun[MQ], lrun[MQ];
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+        mrun[mq] = NEG_BIG; lrun[mq] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) o[mq][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int nkb = (p.keys + 63) >> 6;
+    for (int kb = w; kb < nkb; kb += WAVES) {
+        const int key0 = kb * 64;
+        f32x4 st[MQ][4];
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) st[mq][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            const int key = min(key0 + nt * 16 + r, p.keys - 1);
+            const bf16_t* kp = p.k + (size_t)key * p.ldk + 8 * g;
+#pragma unroll
+            for (int kd = 0; kd < 8; ++kd) {
+                const bf16x8 kf = *(const bf16x8*)(kp + kd * 32);
+#pragma unroll
+                for (int mq = 0; mq < MQ; ++mq) st[mq][nt] = mfma16(kf, qf[mq][kd], st[mq][nt]);
+            }
+        }
+        bf16x8 pb[MQ][2];
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq) {
+            const int row = m0 + mq * 16 + r;
+            float mx = NEG_BIG;
+            bool vis[4][4];
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int key = key0 + nt * 16 + 4 * g + v;
+                    bool ok = key < p.keys;
+                    if (key < p.prefix_alloc) ok = ok && key < vl;
+                    else ok = ok && (row >= p.state_rows || key == p.prefix_alloc);
+                    vis[nt][v] = ok;
+                    const float s = ok ? st[mq][nt][v] * p.scale : NEG_BIG;
+                    st[mq][nt][v] = s;
+                    mx = fmaxf(mx, s);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float mnew = fmaxf(mrun[mq], mx);
+            const float alpha = __expf(mrun[mq] - mnew);
+            float sum = 0.f;
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float e = vis[nt][v] ? __expf(st[mq][nt][v] - mnew) : 0.f;
+                    st[mq][nt][v] = e;
+                    sum += e;
+                }
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            lrun[mq] = lrun[mq] * alpha + sum;
+            mrun[mq] = mnew;
+#pragma unroll
+            for (int dt = 0; dt < 16; ++dt) o[mq][dt] *= alpha;
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) pb[mq][kk] = cat44(pack4(st[mq][2 * kk]), pack4(st[mq][2 * kk + 1]));
+        }
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) {
+            const bf16_t* vp = p.vt + (size_t)(dt * 16 + r) * p.ldvt + key0 + 4 * g;
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                const bf16x8 vf = cat44(load4(vp + kk * 32), load4(vp + kk * 32 + 16));
+#pragma unroll
+                for (int mq = 0; mq < MQ; ++mq) o[mq][dt] = mfma16(vf, pb[mq][kk], o[mq][dt]);
+            }
+        }
+    }
+
+    // ---- merge the key splits of the WAVES waves ----
+    if (g == 0) {
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq) ms[(w * MQ + mq) * 16 + r] = mrun[mq];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+        float mg = NEG_BIG;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) mg = fmaxf(mg, ms[(ww * MQ + mq) * 16 + r]);
+        const float sc = __expf(mrun[mq] - mg);
+        lrun[mq] *= sc;
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) o[mq][dt] *= sc;
+        if (g == 0) ls[(w * MQ + mq) * 16 + r] = lrun[mq];
+    }
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+        __syncthreads();                       // ls written / previous obuf round consumed
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) obuf[((size_t)w * 16 + dt) * 64 + lane] = o[mq][dt];
+        __syncthreads();
+        float lt = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) lt += ls[(ww * MQ + mq) * 16 + r];
+        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+        const int row = m0 + mq * 16 + r;
+        for (int dt = w; dt < 16; dt += WAVES) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ww = 0; ww < WAVES; ++ww) t += obuf[((size_t)ww * 16 + dt) * 64 + lane];
+            if (row < p.rows) store4(p.out + (size_t)row * p.ldo + dt * 16 + 4 * g, pack4(t * inv));
+        }
+    }
+}
+
+// SigLIP: qk [views*256][2304] = Q(16 x 72) | K(16 x 72), vt [views*16][80][256], out [views*256][1152].
+// One wave per 16 query rows over all 256 keys; 4 waves per workgroup.
+__global__ __launch_bounds__(256)
+void vision_attn_kernel(const bf16_t* __restrict__ qk, const bf16_t* __restrict__ vt, bf16_t* __restrict__ out) {
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int g = lane >> 4, r = lane & 15;
+    const int blk = blockIdx.x;                  // (view*16 + head)*4 + quarter
+    const int quarter = blk & 3, vh = blk >> 2, head = vh & 15, view = vh >> 4;
+    const int row = view * 256 + quarter * 64 + w * 16 + r;       // query token (global row)
+    const float scale = 0.11785113019775792f;                      // 1 / sqrt(72)
+    const bf16x8 zero8 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    bf16x8 qf[3];
+    {
+        const bf16_t* qp = qk + (size_t)row * 2304 + head * 72 + 8 * g;
+        qf[0] = *(const bf16x8*)qp;
+        qf[1] = *(const bf16x8*)(qp + 32);
+        qf[2] = (g == 0) ? *(const bf16x8*)(qp + 64) : zero8;
+    }
+    f32x4 o[5];
+#pragma unroll
+    for (int dt = 0; dt < 5; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float mrun = NEG_BIG, lrun = 0.f;
+    const bf16_t* vbase = vt + (size_t)vh * 80 * 256;
+
+    for (int kb = 0; kb < 4; ++kb) {
+        const int key0 = kb * 64;
+        f32x4 st[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            st[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const bf16_t* kp = qk + (size_t)(view * 256 + key0 + nt * 16 + r) * 2304 + 1152 + head * 72 + 8 * g;
+            st[nt] = mfma16(*(const bf16x8*)kp, qf[0], st[nt]);
+            st[nt] = mfma16(*(const bf16x8*)(kp + 32), qf[1], st[nt]);
+            const bf16x8 k2 = (g == 0) ? *(const bf16x8*)(kp + 64) : zero8;
+            st[nt] = mfma16(k2, qf[2], st[nt]);
+        }
+        float mx = NEG_BIG;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) { st[nt][v] *= scale; mx = fmaxf(mx, st[nt][v]); }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mnew = fmaxf(mrun, mx);
+        const float alpha = __expf(mrun - mnew);
+        float sum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) { st[nt][v] = __expf(st[nt][v] - mnew); sum += st[nt][v]; }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        lrun = lrun * alpha + sum;
+        mrun = mnew;
+        bf16x8 pb[2];
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) pb[kk] = cat44(pack4(st[2 * kk]), pack4(st[2 * kk + 1]));
+#pragma unroll
+        for (int dt = 0; dt < 5; ++dt) {
+            o[dt] *= alpha;
+            const bf16_t* vp = vbase + (size_t)(dt * 16 + r) * 256 + key0 + 4 * g;
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+                o[dt] = mfma16(cat44(load4(vp + kk * 32), load4(vp + kk * 32 + 16)), pb[kk], o[dt]);
+        }
+    }
+    const float inv = 1.0f / lrun;
+#pragma unroll
+    for (int dt = 0; dt < 5; ++dt) {
+        const int d = dt * 16 + 4 * g;
+        if (d < 72) store4(out + (size_t)row * 1152 + head * 72 + d, pack4(o[dt] * inv));
+    }
+}
+
+template <int WAVES, int MQ>
+int launch_mqa_inst(const AttnP& p, hipStream_t s) {
+    const size_t smem = (size_t)WAVES * 16 * 64 * 16 + (size_t)2 * WAVES * MQ * 16 * 4;
+    auto kern = mqa_kernel<WAVES, MQ>;
+    if (smem > 65536) {
+        static bool done = false;
+        if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
+    }
+    const int blocks = (p.rows + 16 * MQ - 1) / (16 * MQ);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(WAVES * 64), smem, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+}
+
+}  // namespace
+
+int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s) {
+    if (p.rows <= 0 || p.keys <= 0 || p.ldvt < ((p.keys + 63) / 64) * 64) return 1;
+    if (waves == 8) return launch_mqa_inst<8, 1>(p, s);
+    if (waves == 4) return launch_mqa_inst<4, 2>(p, s);
+    return 2;
+}
+
+void launch_vision_attention(const bf16_t* qk, const bf16_t* vt, bf16_t* out, int views, hipStream_t s) {
+    hipLaunchKernelGGL(vision_attn_kernel, dim3(views * 16 * 4), dim3(256), 0, s, qk, vt, out);
+}

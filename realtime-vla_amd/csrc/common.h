@@ -1,0 +1,55 @@
+// Shared device helpers for the gfx950 kernels: bf16 vector types, MFMA wrapper,
+// packing, activation functions and the XCD-aware block remap.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define RTVLA_DEVICE __device__ __forceinline__
+
+// D[16x16] += A[16x32] * B[32x16] on one wavefront.
+// Operand layout (lane l, g = l / 16, r = l % 16):
+//   a[j] = A[r][8 g + j], b[j] = B[8 g + j][r], d[v] = D[4 g + v][r].
+RTVLA_DEVICE f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+RTVLA_DEVICE float bf2f(bf16_t x) { return (float)x; }
+RTVLA_DEVICE bf16_t f2bf(float x) { return (bf16_t)x; }
+RTVLA_DEVICE float round_bf16(float x) { return (float)(bf16_t)x; }
+
+RTVLA_DEVICE bf16x4 pack4(float a, float b, float c, float d) {
+    bf16x4 r;
+    r[0] = (bf16_t)a; r[1] = (bf16_t)b; r[2] = (bf16_t)c; r[3] = (bf16_t)d;
+    return r;
+}
+RTVLA_DEVICE bf16x4 pack4(f32x4 v) { return pack4(v[0], v[1], v[2], v[3]); }
+
+RTVLA_DEVICE bf16x4 load4(const bf16_t* p) { return *(const bf16x4*)p; }
+RTVLA_DEVICE void store4(bf16_t* p, bf16x4 v) { *(bf16x4*)p = v; }
+
+RTVLA_DEVICE float sigmoidf_fast(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// tanh-approximated GELU written as a * sigmoid(2 sqrt(2/pi) (a + 0.044715 a^3))
+RTVLA_DEVICE float gelu_tanh(float a) {
+    return a * sigmoidf_fast(1.5957691216057308f * a * (1.0f + 0.044715f * a * a));
+}
+RTVLA_DEVICE float siluf(float a) { return a * sigmoidf_fast(a); }
+
+// The hardware dispatcher deals consecutive workgroup ids round-robin over the 8 XCDs
+// (each with a private L2).  Map the hardware id to a logical id so that consecutive
+// logical ids share an XCD; callers make tiles that share an operand consecutive.
+RTVLA_DEVICE int xcd_remap(int bid, int total) {
+    const int q = total >> 3, r = total & 7;
+    const int xcd = bid & 7, idx = bid >> 3;
+    return xcd * q + (xcd < r ? xcd : r) + idx;
+}
+
+RTVLA_DEVICE float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}

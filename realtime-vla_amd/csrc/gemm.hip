@@ -1,0 +1,246 @@
+// Large-M bf16 GEMM on MFMA for the SigLIP and Gemma-prefix layers
+// (replaces the Triton GEMM family of /root/reference/pi0_infer.py:5-346, :664-691, :777-810).
+//
+// out[M][N] = epilogue(A[M][K] * W[K][N]).  The activations A are staged through LDS in MFMA
+// operand-fragment order (each wave reads whole 1 KB fragments with ds_read_b128, conflict
+// free) and are shared by all waves of the workgroup; the weights are read straight from
+// their pre-tiled layout in HBM into registers (one coalesced 1 KB load per fragment, no LDS
+// round trip), each wave owning its own column tiles.  The product is computed transposed
+// (weights as the MFMA A operand) so that every lane ends up with 4 consecutive output columns
+// of one row: 8-byte packed stores, and RoPE pairs / GeGLU partners sit in the same lane.
+#include "kernels.h"
+
+namespace {
+
+template <int EPI> struct EpiTraits { static constexpr bool dual = (EPI == EPI_GEGLU); };
+
+template <int WN, int MT, int NT, int EPI>
+__global__ __launch_bounds__(WN * 64)
+void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int stages_per_split) {
+    constexpr int NTH = WN * 64;
+    constexpr int BM = MT * 16;
+    constexpr int A_CHUNKS = BM * 8;                       // 16-byte chunks per 64-wide K stage
+    constexpr int AIT = (A_CHUNKS + NTH - 1) / NTH;
+    constexpr int STAGE_ELEMS = BM * 64;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    bf16_t* lds = (bf16_t*)smem_raw;
+
+    const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
+    const int g = lane >> 4, r = lane & 15;
+
+    const int total = m_blocks * n_blocks * p.nsplit;
+    const int lid = xcd_remap(blockIdx.x, total);
+    const int split = lid / (m_blocks * n_blocks);
+    const int rem = lid - split * (m_blocks * n_blocks);
+    const int n_blk = rem / m_blocks;
+    const int m_blk = rem - n_blk * m_blocks;
+    const int m0 = m_blk * BM;
+    const int s_begin = split * stages_per_split;
+    const int s_end = min(s_begin + stages_per_split, stages_total);
+
+    // column tiles of this wave
+    constexpr int HALF = EpiTraits<EPI>::dual ? NT / 2 : NT;
+    int tile_of[NT];
+    const bf16_t* bptr[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int t = (n_blk * WN + wn) * HALF + (j % HALF);
+        tile_of[j] = t;
+        const bf16_t* base = (EpiTraits<EPI>::dual && j >= HALF) ? p.B1 : p.B0;
+        const int tc = min(t, p.N16 - 1);
+        bptr[j] = base + (size_t)tc * p.K32p * 512 + lane * 8;
+    }
+    // m-tiles of this block that hold valid rows
+    const int mt_valid = min(MT, (p.M - m0 + 15) >> 4);
+
+    f32x4 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    uint4 areg[AIT];
+    bf16x8 breg0[NT][2], breg1[NT][2];
+
+    auto load_a = [&](int s) {
+#pragma unroll
+        for (int it = 0; it < AIT; ++it) {
+            const int c = it * NTH + tid;
+            if (A_CHUNKS % NTH == 0 || c < A_CHUNKS) {
+                const int row = c >> 3, kc = c & 7;
+                const int gr = min(m0 + row, p.a_rows - 1);
+                areg[it] = *(const uint4*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
+            }
+        }
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < AIT; ++it) {
+            const int c = it * NTH + tid;
+            if (A_CHUNKS % NTH == 0 || c < A_CHUNKS) {
+                const int row = c >> 3, kc = c & 7;
+                const int off = ((((row >> 4) * 2 + (kc >> 2)) * 64) + (row & 15) + 16 * (kc & 3)) * 8;
+                *(uint4*)(lds + buf * STAGE_ELEMS + off) = areg[it];
+            }
+        }
+    };
+    auto load_b = [&](int s, bf16x8 (&br)[NT][2]) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+                br[j][kk] = *(const bf16x8*)(bptr[j] + (size_t)(s * 2 + kk) * 512);
+    };
+    auto compute = [&](int buf, bf16x8 (&br)[NT][2]) {
+        const bf16_t* base = lds + buf * STAGE_ELEMS + lane * 8;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                if (i < mt_valid) {
+                    const bf16x8 a = *(const bf16x8*)(base + (i * 2 + kk) * 512);
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) acc[i][j] = mfma16(br[j][kk], a, acc[i][j]);
+                }
+            }
+        }
+    };
+
+    if (s_begin < s_end) {
+        load_a(s_begin);
+        load_b(s_begin, breg0);
+        store_a(0);
+        __syncthreads();
+        for (int s = s_begin; s < s_end; s += 2) {
+            const bool more1 = s + 1 < s_end;
+            if (more1) { load_a(s + 1); load_b(s + 1, breg1); }
+            compute(0, breg0);
+            if (more1) store_a(1);
+            __syncthreads();
+            if (!more1) break;
+            const bool more2 = s + 2 < s_end;
+            if (more2) { load_a(s + 2); load_b(s + 2, breg0); }
+            compute(1, breg1);
+            if (more2) store_a(0);
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: lane (g, r) holds rows m = m0 + 16 i + r, columns n = 16 tile + 4 g + v ----
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = m0 + i * 16 + r;
+        if (i >= mt_valid || m >= p.M) continue;
+#pragma unroll
+        for (int j = 0; j < HALF; ++j) {
+            const int t = tile_of[j];
+            if (t >= p.N16) continue;
+            const int n0 = t * 16 + 4 * g;
+            f32x4 v = acc[i][j];
+            if constexpr (EPI == EPI_PARTIAL) {
+                *(f32x4*)(p.partial + (size_t)split * p.pstride + (size_t)m * p.ldp + n0) = v;
+            } else if constexpr (EPI == EPI_GEGLU) {
+                const f32x4 u = acc[i][j + HALF];
+                store4(p.out + (size_t)m * p.ldo + n0,
+                       pack4(gelu_tanh(v[0]) * u[0], gelu_tanh(v[1]) * u[1], gelu_tanh(v[2]) * u[2], gelu_tanh(v[3]) * u[3]));
+            } else if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_PATCH) {
+                const bf16x4 b = load4(p.bias + n0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += bf2f(b[e]);
+                if constexpr (EPI == EPI_PATCH) {
+                    const bf16x4 rs = load4(p.res + (size_t)(m % p.res_mod) * p.ldr + n0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += bf2f(rs[e]);
+                }
+                if constexpr (EPI == EPI_BIAS_GELU) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+                }
+                store4(p.out + (size_t)m * p.ldo + n0, pack4(v));
+            } else if constexpr (EPI == EPI_QKV_ROPE) {
+                // the reference rounds the accumulator to bf16 before the rotation (pi0_infer.py:793)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = round_bf16(v[e]);
+                if (n0 < 2304) {
+                    const bf16x4 cs = load4(p.rope + (size_t)m * 256 + (n0 & 255));
+                    const float c0 = bf2f(cs[0]), s0 = bf2f(cs[1]), c1 = bf2f(cs[2]), s1 = bf2f(cs[3]);
+                    const f32x4 w = v;
+                    v[0] = w[0] * c0 - w[1] * s0; v[1] = w[1] * c0 + w[0] * s0;
+                    v[2] = w[2] * c1 - w[3] * s1; v[3] = w[3] * c1 + w[2] * s1;
+                    if (n0 < 2048) store4(p.q + (size_t)m * 2048 + n0, pack4(v));
+                    else store4(p.k + (size_t)m * 256 + (n0 - 2048), pack4(v));
+                } else {
+                    const int d = n0 - 2304;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) p.vt[(size_t)(d + e) * p.ldvt + m] = f2bf(v[e]);
+                }
+            } else if constexpr (EPI == EPI_VIS_QKV) {
+                const bf16x4 b = load4(p.bias + n0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += bf2f(b[e]);
+                if (n0 < 2304) {
+                    store4(p.out + (size_t)m * p.ldo + n0, pack4(v));
+                } else {
+                    const int c = n0 - 2304, head = c / 72, d = c - head * 72;
+                    const int view = m >> 8, tok = m & 255;
+                    bf16_t* dst = p.vt + ((size_t)(view * 16 + head) * 80 + d) * 256 + tok;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dst[(size_t)e * 256] = f2bf(v[e]);
+                }
+            }
+        }
+    }
+}
+
+template <int WN, int MT, int NT, int EPI>
+int launch_cfg(const GemmP& p, hipStream_t s) {
+    constexpr int BM = MT * 16;
+    constexpr int HALF = EpiTraits<EPI>::dual ? NT / 2 : NT;
+    const int m_blocks = (p.M + BM - 1) / BM;
+    const int n_blocks = (p.N16 + WN * HALF - 1) / (WN * HALF);
+    const int stages_total = p.K32p / 2;
+    const int nsplit = p.nsplit < 1 ? 1 : p.nsplit;
+    const int sps = (stages_total + nsplit - 1) / nsplit;
+    if ((nsplit - 1) * sps >= stages_total) return 3;      // an empty split would leave its partial unwritten
+    GemmP q = p; q.nsplit = nsplit;
+    const size_t smem = (size_t)2 * BM * 64 * sizeof(bf16_t);
+    auto kern = gemm_mfma_kernel<WN, MT, NT, EPI>;
+    if (smem > 65536) {
+        static bool done = false;
+        if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
+    }
+    hipLaunchKernelGGL(kern, dim3(m_blocks * n_blocks * nsplit), dim3(WN * 64), smem, s, q, m_blocks, n_blocks, stages_total, sps);
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+}
+
+template <int EPI>
+int launch_epi(const GemmP& p, int tile, hipStream_t s) {
+    switch (tile) {
+        case TILE_256x256: return launch_cfg<4, 16, 4, EPI>(p, s);
+        case TILE_208x256: return launch_cfg<4, 13, 4, EPI>(p, s);
+        case TILE_128x256: return launch_cfg<4, 8, 4, EPI>(p, s);
+        case TILE_128x128: return launch_cfg<4, 8, 2, EPI>(p, s);
+        case TILE_64x256:  return launch_cfg<4, 4, 4, EPI>(p, s);
+    }
+    return 2;
+}
+
+}  // namespace
+
+int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {256, 208, 128, 128, 64}; return v[tile]; }
+int gemm_tile_bn(int tile) { static const int v[TILE_COUNT] = {256, 256, 256, 128, 256}; return v[tile]; }
+
+int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {
+    if (p.M <= 0 || p.N16 <= 0 || p.K32p <= 0 || (p.K32p & 1) || p.a_rows <= 0) return 1;
+    if (epi != EPI_PARTIAL && p.nsplit > 1) return 1;
+    switch (epi) {
+        case EPI_BIAS:      return launch_epi<EPI_BIAS>(p, tile, s);
+        case EPI_BIAS_GELU: return launch_epi<EPI_BIAS_GELU>(p, tile, s);
+        case EPI_PATCH:     return launch_epi<EPI_PATCH>(p, tile, s);
+        case EPI_GEGLU:     return launch_epi<EPI_GEGLU>(p, tile, s);
+        case EPI_PARTIAL:   return launch_epi<EPI_PARTIAL>(p, tile, s);
+        case EPI_QKV_ROPE:  return launch_epi<EPI_QKV_ROPE>(p, tile, s);
+        case EPI_VIS_QKV:   return launch_epi<EPI_VIS_QKV>(p, tile, s);
+    }
+    return 2;
+}

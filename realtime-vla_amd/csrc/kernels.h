@@ -1,0 +1,111 @@
+// Host-side launch interface of the kernel files.  Every launcher enqueues on the given
+// stream, allocates nothing and never synchronises, so all of them can be recorded
+// into a HIP graph.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+#include "common.h"
+
+// ----- pre-tiled weights ------------------------------------------------------------
+// A weight W[K][N] (row-major, "in x out") is re-laid out once as MFMA operand fragments:
+// tile (nb, kb) holds the 16 columns nb*16.. and 32 rows kb*32.. as 64 lanes x 8 bf16,
+// lane l = 16 g + r carrying W[kb*32 + 8 g + j][nb*16 + r], j = 0..7.  Tiles are stored
+// [nb][kb] so that one column block streams contiguously along K.  K is padded to a
+// multiple of 64 and N to a multiple of 16 with zeros.
+static inline int k32_padded(int K) { return ((K + 63) / 64) * 2; }
+static inline int n16_tiles(int N) { return (N + 15) / 16; }
+static inline size_t tiled_elems(int K, int N) { return (size_t)n16_tiles(N) * k32_padded(K) * 512; }
+
+void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, hipStream_t s);
+
+// ----- large-M MFMA GEMM --------------------------------------------------------------
+enum GemmEpilogue {
+    EPI_BIAS = 0,      // out = acc + bias
+    EPI_BIAS_GELU,     // out = gelu_tanh(acc + bias)
+    EPI_PATCH,         // out = acc + bias + res[row % res_mod]
+    EPI_GEGLU,         // out = gelu_tanh(acc(B0)) * acc(B1)
+    EPI_PARTIAL,       // fp32 split-K partial
+    EPI_QKV_ROPE,      // Gemma prefix: bf16 -> interleaved RoPE on Q,K -> Q / K cache / transposed V cache
+    EPI_VIS_QKV,       // SigLIP: +bias, Q|K row-major, V transposed per (view, head)
+};
+
+struct GemmP {
+    const bf16_t* A; int lda; int a_rows;      // activations, rows clamped to a_rows - 1
+    const bf16_t* B0; const bf16_t* B1;        // pre-tiled weights
+    int M, N16, K32p;                          // valid rows, column tiles, padded k32 count
+    int nsplit;                                // split-K factor (EPI_PARTIAL only when > 1)
+    bf16_t* out; int ldo;
+    const bf16_t* bias;
+    const bf16_t* res; int ldr; int res_mod;
+    float* partial; int ldp; size_t pstride;   // [split][row][ldp]
+    const bf16_t* rope;                        // [row][256] = cos0 sin0 cos1 sin1 ...
+    bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt;
+};
+// tile configuration: 0 = 256x256 block (4 waves x 16x4 tiles), 1 = 208x256, 2 = 128x256, 3 = 128x128 (2x2 waves? no: 4 waves x 8x2)
+enum GemmTile { TILE_256x256 = 0, TILE_208x256, TILE_128x256, TILE_128x128, TILE_64x256, TILE_COUNT };
+int gemm_tile_bm(int tile);
+int gemm_tile_bn(int tile);
+int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s);
+
+// ----- split-K reduce + bias + residual (+ gate) + normalisation -----------------------
+enum NormMode { NORM_NONE = 0, NORM_RMS, NORM_LAYER };
+struct ReduceP {
+    const float* partial; size_t pstride; int ldp; int nsplit;   // nsplit may be 0
+    const bf16_t* bias; const bf16_t* res; int ldr;
+    bf16_t* x; int ldx;                         // new residual stream (may be null)
+    bf16_t* xn; int ldxn;                       // normalised copy (may be null)
+    int M, N;
+    int norm; const bf16_t* nw; const bf16_t* nb; float eps;
+};
+int launch_reduce(const ReduceP& p, hipStream_t s);
+
+// ----- skinny (M <= 64) weight-streaming GEMM ---------------------------------------------
+enum SkinnyEpilogue {
+    SK_BIAS = 0,       // out = acc + bias
+    SK_BIAS_SILU,      // out = silu(acc + bias)
+    SK_RES,            // out += acc (* gate[col])
+    SK_QKV_ROPE,       // RoPE + scatter to Q / K cache rows / transposed V cache columns
+    SK_GEGLU,          // out = gelu_tanh(acc(B0)) * acc(B1)
+};
+enum SkinnyNorm { SN_NONE = 0, SN_RMS, SN_ADARMS };
+struct SkinnyP {
+    const bf16_t* A; int lda; int M;           // valid rows (<= 64)
+    const bf16_t* B0; const bf16_t* B1; int K; int N16; int K32p;
+    int norm; const bf16_t* style;             // SN_ADARMS: [scale | shift | gate] each K wide
+    float eps;
+    bf16_t* out; int ldo;
+    const bf16_t* bias; const bf16_t* gate;    // per-column
+    const bf16_t* rope;                        // [row][256]
+    bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt; int kv_row0;
+};
+int launch_skinny(const SkinnyP& p, int epi, hipStream_t s);
+
+// out[m][n] = act(bias[n] + sum_k x[m][k] W[k][n]) for tiny K (<= 64), W in its original layout
+void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t* bias, bf16_t* out, int ldo,
+                         int M, int K, int N, int act_silu, hipStream_t s);
+
+// ----- attention --------------------------------------------------------------------------
+struct AttnP {
+    const bf16_t* q; int ldq;        // [rows][ldq]
+    const bf16_t* k; int ldk;        // [keys][ldk]
+    const bf16_t* vt; int ldvt;      // [d][ldvt] (keys contiguous)
+    bf16_t* out; int ldo;            // [rows][ldo]
+    int rows, keys;
+    float scale;
+    // masking: key j is visible to row r iff
+    //   j < prefix_alloc ? j < *valid_len (or prefix_alloc if valid_len == null)
+    //                    : (r >= state_rows || j == prefix_alloc)
+    int prefix_alloc; const int* valid_len; int state_rows;
+};
+int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s);
+// SigLIP attention: qk [views*256][2304] (Q | K, 16 heads x 72), vt [views*16][80][256]
+void launch_vision_attention(const bf16_t* qk, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);
+
+// ----- small helpers ------------------------------------------------------------------------
+void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hipStream_t s);
+void launch_rope_table(bf16_t* table, const int* start_minus_one_ptr, int start, int count, hipStream_t s);
+void launch_copy_rows(const bf16_t* src, int lds, bf16_t* dst, int ldd, int rows, int cols, hipStream_t s);
+void launch_fill_zero(void* p, size_t bytes, hipStream_t s);
+void launch_scale_inplace(bf16_t* p, size_t n, float f, hipStream_t s);
+void launch_copy_bytes(const void* src, void* dst, size_t bytes, hipStream_t s);

@@ -1,0 +1,224 @@
+// Bandwidth-trivial kernels around the GEMMs: weight pre-tiling, split-K reduce fused with
+// bias / residual / LayerNorm / RMSNorm, patch im2col, tiny-K linear layers, RoPE tables.
+#include "kernels.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// W[K][N] -> MFMA fragment tiles [nb][kb][lane][8] (see kernels.h)
+__global__ void pretile_kernel(const bf16_t* __restrict__ W, int K, int N, bf16_t* __restrict__ out, int K32p, size_t chunks) {
+    const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= chunks) return;
+    const int lane = (int)(c & 63);
+    const size_t tile = c >> 6;
+    const int kb = (int)(tile % K32p), nb = (int)(tile / K32p);
+    const int n = nb * 16 + (lane & 15);
+    const int k0 = kb * 32 + 8 * (lane >> 4);
+    bf16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int k = k0 + j;
+        v[j] = (n < N && k < K) ? W[(size_t)k * N + n] : (bf16_t)0.0f;
+    }
+    *(bf16x8*)(out + c * 8) = v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// One workgroup per row: x = bf16(res + bias + sum_s partial[s]); optional normalised copy.
+// Replaces merge_split_k_bias_res + layer_norm_small_kernel / rms_norm_kernel
+// (/root/reference/pi0_infer.py:325-346, :366-382, :648-663).
+template <int NORM>
+__global__ __launch_bounds__(256)
+void reduce_kernel(ReduceP p) {
+    __shared__ float red[8];
+    const int m = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int nq = p.N >> 2;                   // float4 groups per row (N <= 2048 -> at most 2 per thread)
+    f32x4 v[2];
+    float s = 0.f;
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int c = tid + it * 256;
+        v[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (c < nq) {
+            const int n0 = c * 4;
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+            for (int sp = 0; sp < p.nsplit; ++sp)
+                a += *(const f32x4*)(p.partial + (size_t)sp * p.pstride + (size_t)m * p.ldp + n0);
+            if (p.bias) { const bf16x4 b = load4(p.bias + n0); for (int e = 0; e < 4; ++e) a[e] += bf2f(b[e]); }
+            if (p.res) { const bf16x4 rr = load4(p.res + (size_t)m * p.ldr + n0); for (int e = 0; e < 4; ++e) a[e] += bf2f(rr[e]); }
+            const bf16x4 xb = pack4(a);
+            if (p.x) store4(p.x + (size_t)m * p.ldx + n0, xb);
+            for (int e = 0; e < 4; ++e) a[e] = bf2f(xb[e]);       // the norm reads the bf16 stream
+            v[it] = a;
+            if (NORM == NORM_RMS) s += a[0] * a[0] + a[1] * a[1] + a[2] * a[2] + a[3] * a[3];
+            else s += a[0] + a[1] + a[2] + a[3];
+        }
+    }
+    if (NORM == NORM_NONE) return;
+    auto block_sum = [&](float x) {
+        x = wave_sum(x);
+        __syncthreads();
+        if ((tid & 63) == 0) red[tid >> 6] = x;
+        __syncthreads();
+        return red[0] + red[1] + red[2] + red[3];
+    };
+    const float tot = block_sum(s);
+    const float inv_n = 1.0f / (float)p.N;
+    if (NORM == NORM_RMS) {
+        const float f = rsqrtf(tot * inv_n + p.eps);
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int c = tid + it * 256;
+            if (c < nq) store4(p.xn + (size_t)m * p.ldxn + c * 4, pack4(v[it] * f));
+        }
+    } else {
+        const float mean = tot * inv_n;
+        float q = 0.f;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int c = tid + it * 256;
+            if (c < nq) for (int e = 0; e < 4; ++e) { const float d = v[it][e] - mean; q += d * d; }
+        }
+        const float var = block_sum(q) * inv_n;
+        const float inv_std = 1.0f / sqrtf(var + p.eps);
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int c = tid + it * 256;
+            if (c < nq) {
+                const int n0 = c * 4;
+                const bf16x4 w = load4(p.nw + n0), b = load4(p.nb + n0);
+                f32x4 o;
+                for (int e = 0; e < 4; ++e) o[e] = (v[it][e] - mean) * inv_std * bf2f(w[e]) + bf2f(b[e]);
+                store4(p.xn + (size_t)m * p.ldxn + n0, pack4(o));
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// NHWC images [v][224][224][3] -> patch rows [v*256][ldp], feature order (dy, dx, c), zero padded
+// to ldp (/root/reference/pi0_infer.py:348-350).
+__global__ void im2col_kernel(const bf16_t* __restrict__ img, bf16_t* __restrict__ out, int ldp, int rows) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int per_row = ldp;
+    if (idx >= rows * per_row) return;
+    const int row = idx / per_row, k = idx - row * per_row;
+    bf16_t val = (bf16_t)0.0f;
+    if (k < 588) {
+        const int view = row >> 8, py = (row >> 4) & 15, px = row & 15;
+        const int dy = k / 42, rem = k - dy * 42;       // rem = dx * 3 + c, contiguous in memory
+        val = img[(((size_t)view * 224 + py * 14 + dy) * 224 + px * 14) * 3 + rem];
+    }
+    out[idx] = val;
+}
+
+// tiny-K linear: one thread per output element, W[K][N] row-major (coalesced over n)
+__global__ void small_linear_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ W,
+                                    const bf16_t* __restrict__ bias, bf16_t* __restrict__ out, int ldo,
+                                    int M, int K, int N, int act_silu) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= M * N) return;
+    const int m = idx / N, n = idx - m * N;
+    float acc = bias ? bf2f(bias[n]) : 0.f;
+    for (int k = 0; k < K; ++k) acc += bf2f(x[(size_t)m * ldx + k]) * bf2f(W[(size_t)k * N + n]);
+    if (act_silu) acc = siluf(acc);
+    out[(size_t)m * ldo + n] = f2bf(acc);
+}
+
+// RoPE table rows [cos_i, sin_i] interleaved for positions pos0 .. pos0 + count - 1, where
+// pos0 = start (+ *dyn_start if the pointer is given).  /root/reference/pi0_infer.py:1319-1335.
+__global__ void rope_table_kernel(bf16_t* __restrict__ table, const int* dyn_start, int start, int count) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= count * 128) return;
+    const int row = idx >> 7, i = idx & 127;
+    const int pos = start + row + (dyn_start ? *dyn_start : 0);
+    const float inv_freq = 1.0f / powf(10000.0f, (float)(2 * i) / 256.0f);
+    const float phase = inv_freq * (float)pos;
+    table[(size_t)row * 256 + 2 * i] = f2bf(cosf(phase));
+    table[(size_t)row * 256 + 2 * i + 1] = f2bf(sinf(phase));
+}
+
+__global__ void copy_rows_kernel(const bf16_t* __restrict__ src, int lds, bf16_t* __restrict__ dst, int ldd, int rows, int cols8) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * cols8) return;
+    const int r = idx / cols8, c = idx - r * cols8;
+    *(uint4*)(dst + (size_t)r * ldd + c * 8) = *(const uint4*)(src + (size_t)r * lds + c * 8);
+}
+
+__global__ void fill_zero_kernel(uint4* p, size_t n16) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) p[i] = uint4{0, 0, 0, 0};
+}
+
+__global__ void copy_bytes_kernel(const uint4* src, uint4* dst, size_t n16) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
+
+__global__ void scale_kernel(bf16_t* p, size_t n, float f) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = f2bf(bf2f(p[i]) * f);
+}
+
+}  // namespace
+
+void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, hipStream_t s) {
+    const int K32p = k32_padded(K);
+    const size_t chunks = (size_t)n16_tiles(N) * K32p * 64;
+    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, K32p, chunks);
+}
+
+int launch_reduce(const ReduceP& p, hipStream_t s) {
+    if (p.M <= 0 || p.N <= 0 || (p.N & 3) || p.N > 2048) return 1;
+    if (p.norm != NORM_NONE && !p.xn) return 1;
+    if (p.norm == NORM_LAYER && (!p.nw || !p.nb)) return 1;
+    switch (p.norm) {
+        case NORM_NONE:  hipLaunchKernelGGL(reduce_kernel<NORM_NONE>, dim3(p.M), dim3(256), 0, s, p); break;
+        case NORM_RMS:   hipLaunchKernelGGL(reduce_kernel<NORM_RMS>, dim3(p.M), dim3(256), 0, s, p); break;
+        case NORM_LAYER: hipLaunchKernelGGL(reduce_kernel<NORM_LAYER>, dim3(p.M), dim3(256), 0, s, p); break;
+        default: return 2;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+}
+
+void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hipStream_t s) {
+    const int rows = views * 256;
+    const int total = rows * ldp;
+    hipLaunchKernelGGL(im2col_kernel, dim3((total + 255) / 256), dim3(256), 0, s, images, patches, ldp, rows);
+}
+
+void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t* bias, bf16_t* out, int ldo,
+                         int M, int K, int N, int act_silu, hipStream_t s) {
+    const int total = M * N;
+    hipLaunchKernelGGL(small_linear_kernel, dim3((total + 255) / 256), dim3(256), 0, s, x, ldx, W, bias, out, ldo, M, K, N, act_silu);
+}
+
+void launch_rope_table(bf16_t* table, const int* dyn_start, int start, int count, hipStream_t s) {
+    const int total = count * 128;
+    hipLaunchKernelGGL(rope_table_kernel, dim3((total + 255) / 256), dim3(256), 0, s, table, dyn_start, start, count);
+}
+
+void launch_copy_rows(const bf16_t* src, int lds, bf16_t* dst, int ldd, int rows, int cols, hipStream_t s) {
+    if (rows <= 0 || cols <= 0) return;
+    const int cols8 = cols / 8;
+    const int total = rows * cols8;
+    hipLaunchKernelGGL(copy_rows_kernel, dim3((total + 255) / 256), dim3(256), 0, s, src, lds, dst, ldd, rows, cols8);
+}
+
+void launch_fill_zero(void* p, size_t bytes, hipStream_t s) {
+    const size_t n16 = bytes / 16;
+    if (!n16) return;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, (uint4*)p, n16);
+}
+
+void launch_copy_bytes(const void* src, void* dst, size_t bytes, hipStream_t s) {
+    const size_t n16 = bytes / 16;
+    if (!n16) return;
+    hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, (const uint4*)src, (uint4*)dst, n16);
+}
+
+void launch_scale_inplace(bf16_t* p, size_t n, float f, hipStream_t s) {
+    if (!n) return;
+    hipLaunchKernelGGL(scale_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, f);
+}

@@ -1,0 +1,716 @@
+// Context, workspace layout, static launch schedule and C ABI (include/rtvla.h) of the
+// Pi0 / Pi05 forward pass.  The schedule restates pi0_model (/root/reference/pi0_infer.py:1232-1236)
+// and pi05_model (/root/reference/pi05_infer.py:525-528) as a fixed list of kernel launches that
+// touch only caller-owned memory, so the whole forward can be captured into one HIP graph.
+#include "../../include/rtvla.h"
+#include "kernels.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace {
+
+struct Tensor {
+    std::string name;
+    int elem = 2;
+    int rank = 0;
+    int64_t shape[4] = {0, 0, 0, 0};
+    bool weight = true;
+    bool required = true;
+    void* ptr = nullptr;
+    bool bound = false;
+    size_t bytes() const { size_t n = elem; for (int i = 0; i < rank; ++i) n *= (size_t)shape[i]; return n; }
+};
+
+struct WsBuf {
+    std::string name;
+    size_t offset = 0;
+    int64_t rows = 0, cols = 0, ld = 0;
+    int elem = 2;
+    size_t bytes() const { return (size_t)rows * ld * elem; }
+};
+
+struct TileChoice { int tile; int nsplit; };
+
+}  // namespace
+
+struct rtvla_ctx {
+    rtvla_dims d;
+    int S_v = 0, S_e = 0, S_d = 0, keys = 0, keys_pad = 0;
+    std::vector<Tensor> tensors;
+    std::map<std::string, int> tindex;
+    std::vector<WsBuf> bufs;
+    std::map<std::string, int> bindex;
+    size_t ws_bytes = 0;
+    size_t act_begin = 0;          // activations start here (cleared at prepare)
+    char* ws = nullptr;
+    bool prepared = false;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::string err;
+    int launches = 0;
+    int status = 0;
+
+    // ---- helpers ----
+    int fail(int code, const std::string& msg) { err = msg; return code; }
+    Tensor& T(const char* n) { return tensors[tindex.at(n)]; }
+    bf16_t* W(const char* n) { return (bf16_t*)tensors[tindex.at(n)].ptr; }
+    bf16_t* W(const char* n, size_t layer_elems, int layer) { return (bf16_t*)tensors[tindex.at(n)].ptr + layer_elems * layer; }
+    template <typename X = bf16_t> X* B(const char* n) { return (X*)(ws + bufs[bindex.at(n)].offset); }
+    const WsBuf& BI(const char* n) const { return bufs[bindex.at(n)]; }
+
+    void add_tensor(const char* name, bool weight, int elem, std::initializer_list<int64_t> shape) {
+        Tensor t; t.name = name; t.weight = weight; t.elem = elem; t.rank = (int)shape.size();
+        int i = 0; for (auto s : shape) t.shape[i++] = s;
+        tindex[name] = (int)tensors.size();
+        tensors.push_back(t);
+    }
+    void add_buf(const char* name, int64_t rows, int64_t cols, int64_t ld, int elem = 2) {
+        WsBuf b; b.name = name; b.rows = rows; b.cols = cols; b.ld = ld; b.elem = elem;
+        b.offset = ws_bytes;
+        ws_bytes += (b.bytes() + 255) & ~(size_t)255;
+        bindex[name] = (int)bufs.size();
+        bufs.push_back(b);
+    }
+    void add_tiled(const char* name, int K, int N, int layers) {
+        add_buf(name, layers, (int64_t)tiled_elems(K, N), (int64_t)tiled_elems(K, N));
+    }
+    bf16_t* TW(const char* n, int layer = 0) { const WsBuf& b = BI(n); return (bf16_t*)(ws + b.offset) + (size_t)b.ld * layer; }
+
+    void note(int rc, const char* what) {
+        ++launches;
+        if (rc != 0 && status == 0) { status = RTVLA_ERR_DEVICE; err = std::string("launch failed: ") + what + " (code " + std::to_string(rc) + ")"; }
+    }
+};
+
+namespace {
+
+constexpr int PATCH_LD = 640;      // 588 patch features padded to a multiple of 64
+constexpr int VHID_LD = 4352;      // 4304 padded to a multiple of 64
+
+// Pick block tile and split-K factor from a coarse cost model: workgroups run in rounds of
+// 256 (one per CU); a workgroup's time is proportional to its valid row tiles x K stages plus a
+// fixed prologue/epilogue; split-K adds the fp32 partial traffic.
+TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable) {
+    static const int tiles[] = {TILE_256x256, TILE_208x256, TILE_128x256, TILE_64x256};
+    static const int splits[] = {1, 2, 3, 4, 6, 8};
+    if (const char* e = getenv("RTVLA_FORCE_TILE")) {
+        TileChoice c{atoi(e), 1};
+        if (const char* s = getenv("RTVLA_FORCE_SPLIT")) if (splittable) c.nsplit = atoi(s);
+        return c;
+    }
+    double best = 1e30; TileChoice bc{TILE_128x256, 1};
+    for (int tile : tiles) {
+        const int bm = gemm_tile_bm(tile);
+        const int bn16 = gemm_tile_bn(tile) / 16 / (dual ? 2 : 1);
+        const int mb = (M + bm - 1) / bm, nb = (ncols16 + bn16 - 1) / bn16;
+        const int mt = (std::min(M, bm) + 15) / 16;
+        for (int sp : splits) {
+            if (sp > 1 && !splittable) break;
+            const int sps = (stages + sp - 1) / sp;
+            if ((sp - 1) * sps >= stages) continue;
+            const int blocks = mb * nb * sp;
+            const int rounds = (blocks + 255) / 256;
+            double t = rounds * (mt * (sps + 1.0) * 4.0 * 2 * 16 / 2400.0 + 1.5);       // us: MFMA cycles at 2.4 GHz + fixed
+            if (splittable) t += (double)sp * M * ncols16 * 16 * 8.0 / 3.0e6;         // fp32 partial write + read at ~3 TB/s
+            if (t < best) { best = t; bc = TileChoice{tile, sp}; }
+        }
+    }
+    return bc;
+}
+
+int build_tables(rtvla_ctx* c) {
+    const rtvla_dims& d = c->d;
+    const int64_t V = d.vision_layers, L = d.llm_layers, v = d.num_views, ch = d.chunk_size;
+    const bool pi05 = d.model == RTVLA_PI05;
+    // ---- tensors that cross the boundary (reference names and shapes) ----
+    c->add_tensor("vision_patch_embedding_w", true, 2, {14, 14, 3, 1152});
+    c->add_tensor("vision_patch_embedding_b", true, 2, {1152});
+    c->add_tensor("vision_position_embedding", true, 2, {256, 1152});
+    c->add_tensor("vision_attn_qkv_w", true, 2, {V, 1152, 3456});
+    c->add_tensor("vision_attn_qkv_b", true, 2, {V, 3456});
+    c->add_tensor("vision_attn_o_w", true, 2, {V, 1152, 1152});
+    c->add_tensor("vision_attn_o_b", true, 2, {V, 1152});
+    c->add_tensor("vision_ffn_up_w", true, 2, {V, 1152, 4304});
+    c->add_tensor("vision_ffn_up_b", true, 2, {V, 4304});
+    c->add_tensor("vision_ffn_down_w", true, 2, {V, 4304, 1152});
+    c->add_tensor("vision_ffn_down_b", true, 2, {V, 1152});
+    c->add_tensor("vision_pre_attn_norm_w", true, 2, {V, 1152});
+    c->add_tensor("vision_pre_attn_norm_b", true, 2, {V, 1152});
+    c->add_tensor("vision_pre_ffn_norm_w", true, 2, {V, 1152});
+    c->add_tensor("vision_pre_ffn_norm_b", true, 2, {V, 1152});
+    c->add_tensor("vision_final_norm_w", true, 2, {1152});
+    c->add_tensor("vision_final_norm_b", true, 2, {1152});
+    c->add_tensor("encoder_multi_modal_projector_w", true, 2, {1152, 2048});
+    c->add_tensor("encoder_multi_modal_projector_b", true, 2, {2048});
+    c->add_tensor("encoder_attn_qkv_w", true, 2, {L, 2048, 2560});
+    c->add_tensor("encoder_attn_o_w", true, 2, {L, 2048, 2048});
+    c->add_tensor("encoder_ffn_gate_w", true, 2, {L, 2048, 16384});
+    c->add_tensor("encoder_ffn_up_w", true, 2, {L, 2048, 16384});
+    c->add_tensor("encoder_ffn_down_w", true, 2, {L, 16384, 2048});
+    if (!pi05) {
+        c->add_tensor("decoder_state_in_proj_w", true, 2, {32, 1024});
+        c->add_tensor("decoder_state_in_proj_b", true, 2, {1024});
+        c->add_tensor("decoder_action_fused_in_proj_w", true, 2, {32, 1024});
+        c->add_tensor("decoder_action_fused_time_biases", true, 2, {10, 1024});
+        c->add_tensor("decoder_action_mlp_w", true, 2, {1024, 1024});
+        c->add_tensor("decoder_action_mlp_b", true, 2, {1024});
+    } else {
+        c->add_tensor("decoder_time_embeds", true, 2, {10, 1024});
+        c->add_tensor("decoder_time_mlp_in_w", true, 2, {1024, 1024});
+        c->add_tensor("decoder_time_mlp_in_b", true, 2, {1024});
+        c->add_tensor("decoder_time_mlp_out_w", true, 2, {1024, 1024});
+        c->add_tensor("decoder_time_mlp_out_b", true, 2, {1024});
+        c->add_tensor("decoder_action_in_proj_w", true, 2, {32, 1024});
+        c->add_tensor("decoder_action_in_proj_b", true, 2, {1024});
+        c->add_tensor("decoder_pre_attn_norm_mod_w", true, 2, {L, 1024, 3072});
+        c->add_tensor("decoder_pre_attn_norm_mod_b", true, 2, {L, 3072});
+        c->add_tensor("decoder_pre_ffn_norm_mod_w", true, 2, {L, 1024, 3072});
+        c->add_tensor("decoder_pre_ffn_norm_mod_b", true, 2, {L, 3072});
+    }
+    c->add_tensor("decoder_attn_qkv_w", true, 2, {L, 1024, 2560});
+    c->add_tensor("decoder_attn_o_w", true, 2, {L, 2048, 1024});
+    c->add_tensor("decoder_ffn_gate_w", true, 2, {L, 1024, 4096});
+    c->add_tensor("decoder_ffn_up_w", true, 2, {L, 1024, 4096});
+    c->add_tensor("decoder_ffn_down_w", true, 2, {L, 4096, 1024});
+    if (!pi05) {
+        c->add_tensor("decoder_action_fused_out_proj_w", true, 2, {1024, 32});
+        c->add_tensor("decoder_action_fused_out_proj_b", true, 2, {32});
+        c->add_tensor("language_embeds", true, 2, {d.prompt_len, 2048});
+    } else {
+        c->add_tensor("decoder_action_out_proj_w", true, 2, {1024, 32});
+        c->add_tensor("decoder_action_out_proj_b", true, 2, {32});
+        c->add_tensor("decoder_final_norm_mod_w", true, 2, {1024, 3072});
+        c->add_tensor("decoder_final_norm_mod_b", true, 2, {3072});
+    }
+    c->add_tensor("observation_images_normalized", false, 2, {v, 224, 224, 3});
+    if (!pi05) c->add_tensor("observation_state_normalized", false, 2, {32});
+    c->add_tensor("diffusion_noise", false, 2, {ch, 32});
+    c->add_tensor("encoder_rope_weights", false, 2, {c->S_e, 256});
+    c->add_tensor("decoder_rope_weights", false, 2, {c->S_d, 256});
+    if (pi05) c->add_tensor("valid_encoder_len", false, 4, {1});
+
+    // ---- workspace: re-tiled weights first, then activations ----
+    c->add_tiled("t_vision_patch_embedding_w", 588, 1152, 1);
+    c->add_tiled("t_vision_attn_qkv_w", 1152, 3456, V);
+    c->add_tiled("t_vision_attn_o_w", 1152, 1152, V);
+    c->add_tiled("t_vision_ffn_up_w", 1152, 4304, V);
+    c->add_tiled("t_vision_ffn_down_w", 4304, 1152, V);
+    c->add_tiled("t_encoder_multi_modal_projector_w", 1152, 2048, 1);
+    c->add_tiled("t_encoder_attn_qkv_w", 2048, 2560, L);
+    c->add_tiled("t_encoder_attn_o_w", 2048, 2048, L);
+    c->add_tiled("t_encoder_ffn_gate_w", 2048, 16384, L);
+    c->add_tiled("t_encoder_ffn_up_w", 2048, 16384, L);
+    c->add_tiled("t_encoder_ffn_down_w", 16384, 2048, L);
+    c->add_tiled("t_decoder_attn_qkv_w", 1024, 2560, L);
+    c->add_tiled("t_decoder_attn_o_w", 2048, 1024, L);
+    c->add_tiled("t_decoder_ffn_gate_w", 1024, 4096, L);
+    c->add_tiled("t_decoder_ffn_up_w", 1024, 4096, L);
+    c->add_tiled("t_decoder_ffn_down_w", 4096, 1024, L);
+    c->add_tiled("t_decoder_out_proj_w", 1024, 32, 1);
+    if (!pi05) {
+        c->add_tiled("t_decoder_action_mlp_w", 1024, 1024, 1);
+    } else {
+        c->add_tiled("t_decoder_time_mlp_in_w", 1024, 1024, 1);
+        c->add_tiled("t_decoder_time_mlp_out_w", 1024, 1024, 1);
+        c->add_tiled("t_decoder_pre_attn_norm_mod_w", 1024, 3072, L);
+        c->add_tiled("t_decoder_pre_ffn_norm_mod_w", 1024, 3072, L);
+        c->add_tiled("t_decoder_final_norm_mod_w", 1024, 3072, 1);
+        c->add_buf("decoder_out_proj_w_scaled", 1024, 32, 32);
+        c->add_buf("decoder_out_proj_b_scaled", 1, 32, 32);
+    }
+    c->act_begin = c->ws_bytes;
+    const int64_t S_v = c->S_v, S_e = c->S_e, S_d = c->S_d;
+    c->add_buf("vision_patches", S_v, PATCH_LD, PATCH_LD);
+    c->add_buf("vision_x", S_v, 1152, 1152);
+    c->add_buf("vision_x_norm", S_v, 1152, 1152);
+    c->add_buf("vision_QK", S_v, 2304, 2304);
+    c->add_buf("vision_Vt", v * 16 * 80, 256, 256);
+    c->add_buf("vision_attn", S_v, 1152, 1152);
+    c->add_buf("vision_hidden", S_v, 4304, VHID_LD);
+    c->add_buf("encoder_x", S_e, 2048, 2048);
+    c->add_buf("encoder_x_norm", S_e, 2048, 2048);
+    c->add_buf("encoder_Q", S_e, 2048, 2048);
+    c->add_buf("encoder_attn", S_e, 2048, 2048);
+    c->add_buf("encoder_hidden", S_e, 16384, 16384);
+    c->add_buf("encoder_K", L * c->keys, 256, 256);
+    c->add_buf("encoder_Vt", L * 256, c->keys, c->keys_pad);
+    c->add_buf("decoder_x", S_d, 1024, 1024);
+    c->add_buf("decoder_x_buf", std::max<int64_t>(ch, 16), 1024, 1024);
+    c->add_buf("decoder_state_buf", 1, 1024, 1024);
+    c->add_buf("decoder_q_buf", S_d, 2048, 2048);
+    c->add_buf("decoder_attn", S_d, 2048, 2048);
+    c->add_buf("decoder_hidden", S_d, 4096, 4096);
+    if (pi05) {
+        c->add_buf("decoder_time_emb", d.num_steps, 1024, 1024);
+        c->add_buf("decoder_style_attn", d.num_steps, L * 3072, L * 3072);
+        c->add_buf("decoder_style_ffn", d.num_steps, L * 3072, L * 3072);
+        c->add_buf("decoder_style_final", d.num_steps, 3072, 3072);
+    }
+    const int64_t pmax = std::max(S_v * 1152, S_e * 2048) * 8;
+    c->add_buf("splitk_partial", 1, pmax, pmax, 4);
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// schedule
+// ------------------------------------------------------------------------------------------------
+struct Sched {
+    rtvla_ctx* c;
+    hipStream_t s;
+    const rtvla_dims& d;
+    bool pi05;
+    Sched(rtvla_ctx* c_, hipStream_t s_) : c(c_), s(s_), d(c_->d), pi05(c_->d.model == RTVLA_PI05) {}
+
+    void gemm(const bf16_t* A, int lda, int a_rows, int M, const bf16_t* B0, const bf16_t* B1, int K, int N, int epi, GemmP extra, const char* what) {
+        GemmP p = extra;
+        p.A = A; p.lda = lda; p.a_rows = a_rows; p.M = M; p.B0 = B0; p.B1 = B1;
+        p.N16 = n16_tiles(N); p.K32p = k32_padded(K);
+        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU, epi == EPI_PARTIAL);
+        p.nsplit = tc.nsplit;
+        if (epi == EPI_PARTIAL) {
+            p.partial = c->B<float>("splitk_partial"); p.ldp = N; p.pstride = (size_t)M * N;
+        }
+        last_split = tc.nsplit;
+        c->note(launch_gemm(p, epi, tc.tile, s), what);
+    }
+    int last_split = 1;
+
+    void reduce(int M, int N, const bf16_t* bias, const bf16_t* res, int ldr, bf16_t* x, int ldx, bf16_t* xn, int ldxn,
+                int norm, const bf16_t* nw, const bf16_t* nb, float eps, int nsplit, const char* what) {
+        ReduceP p{};
+        p.partial = c->B<float>("splitk_partial"); p.pstride = (size_t)M * N; p.ldp = N; p.nsplit = nsplit;
+        p.bias = bias; p.res = res; p.ldr = ldr; p.x = x; p.ldx = ldx; p.xn = xn; p.ldxn = ldxn;
+        p.M = M; p.N = N; p.norm = norm; p.nw = nw; p.nb = nb; p.eps = eps;
+        c->note(launch_reduce(p, s), what);
+    }
+
+    void vision_embed() {
+        const int S_v = c->S_v;
+        launch_im2col(c->W("observation_images_normalized"), c->B("vision_patches"), PATCH_LD, d.num_views, s); c->note(0, "im2col");
+        GemmP e{}; e.out = c->B("vision_x"); e.ldo = 1152; e.bias = c->W("vision_patch_embedding_b");
+        e.res = c->W("vision_position_embedding"); e.ldr = 1152; e.res_mod = 256;
+        gemm(c->B("vision_patches"), PATCH_LD, S_v, S_v, c->TW("t_vision_patch_embedding_w"), nullptr, 588, 1152, EPI_PATCH, e, "patch embed");
+        reduce(S_v, 1152, nullptr, c->B("vision_x"), 1152, nullptr, 0, c->B("vision_x_norm"), 1152, NORM_LAYER,
+               c->W("vision_pre_attn_norm_w"), c->W("vision_pre_attn_norm_b"), 1e-5f, 0, "vision LN0");
+    }
+
+    void vision_layer(int i) {
+        const int S_v = c->S_v, V = d.vision_layers;
+        GemmP e{}; e.out = c->B("vision_QK"); e.ldo = 2304; e.bias = c->W("vision_attn_qkv_b", 3456, i); e.vt = c->B("vision_Vt");
+        gemm(c->B("vision_x_norm"), 1152, S_v, S_v, c->TW("t_vision_attn_qkv_w", i), nullptr, 1152, 3456, EPI_VIS_QKV, e, "vision qkv");
+        launch_vision_attention(c->B("vision_QK"), c->B("vision_Vt"), c->B("vision_attn"), d.num_views, s); c->note(0, "vision attn");
+        gemm(c->B("vision_attn"), 1152, S_v, S_v, c->TW("t_vision_attn_o_w", i), nullptr, 1152, 1152, EPI_PARTIAL, GemmP{}, "vision o");
+        reduce(S_v, 1152, c->W("vision_attn_o_b", 1152, i), c->B("vision_x"), 1152, c->B("vision_x"), 1152, c->B("vision_x_norm"), 1152,
+               NORM_LAYER, c->W("vision_pre_ffn_norm_w", 1152, i), c->W("vision_pre_ffn_norm_b", 1152, i), 1e-5f, last_split, "vision o reduce");
+        GemmP u{}; u.out = c->B("vision_hidden"); u.ldo = VHID_LD; u.bias = c->W("vision_ffn_up_b", 4304, i);
+        gemm(c->B("vision_x_norm"), 1152, S_v, S_v, c->TW("t_vision_ffn_up_w", i), nullptr, 1152, 4304, EPI_BIAS_GELU, u, "vision up");
+        gemm(c->B("vision_hidden"), VHID_LD, S_v, S_v, c->TW("t_vision_ffn_down_w", i), nullptr, 4304, 1152, EPI_PARTIAL, GemmP{}, "vision down");
+        const bool last = i == V - 1;
+        const bf16_t* nw = last ? c->W("vision_final_norm_w") : c->W("vision_pre_attn_norm_w", 1152, i + 1);
+        const bf16_t* nb = last ? c->W("vision_final_norm_b") : c->W("vision_pre_attn_norm_b", 1152, i + 1);
+        reduce(S_v, 1152, c->W("vision_ffn_down_b", 1152, i), c->B("vision_x"), 1152, c->B("vision_x"), 1152, c->B("vision_x_norm"), 1152,
+               NORM_LAYER, nw, nb, 1e-5f, last_split, "vision down reduce");
+    }
+
+    void project() {
+        const int S_v = c->S_v, S_e = c->S_e;
+        GemmP e{}; e.out = c->B("encoder_x"); e.ldo = 2048; e.bias = c->W("encoder_multi_modal_projector_b");
+        gemm(c->B("vision_x_norm"), 1152, S_v, S_v, c->TW("t_encoder_multi_modal_projector_w"), nullptr, 1152, 2048, EPI_BIAS, e, "projector");
+        if (!pi05 && d.prompt_len > 0) {
+            launch_copy_rows(c->W("language_embeds"), 2048, c->B("encoder_x") + (size_t)S_v * 2048, 2048, d.prompt_len, 2048, s);
+            c->note(0, "prompt rows");
+        }
+        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, nullptr, 0, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, 0, "prefix rms0");
+    }
+
+    bf16_t* Kc(int i) { return c->B("encoder_K") + (size_t)i * c->keys * 256; }
+    bf16_t* Vt(int i) { return c->B("encoder_Vt") + (size_t)i * 256 * c->keys_pad; }
+    const int* valid_len() { return pi05 ? (const int*)c->tensors[c->tindex.at("valid_encoder_len")].ptr : nullptr; }
+
+    void prefix_layer(int i) {
+        const int S_e = c->S_e, L = d.llm_layers;
+        GemmP e{}; e.rope = c->W("encoder_rope_weights"); e.q = c->B("encoder_Q"); e.k = Kc(i); e.vt = Vt(i); e.ldvt = c->keys_pad;
+        gemm(c->B("encoder_x_norm"), 2048, S_e, S_e, c->TW("t_encoder_attn_qkv_w", i), nullptr, 2048, 2560, EPI_QKV_ROPE, e, "prefix qkv");
+        if (i == L - 1) return;                      // the last layer only fills the KV cache
+        AttnP a{};
+        a.q = c->B("encoder_Q"); a.ldq = 256; a.k = Kc(i); a.ldk = 256; a.vt = Vt(i); a.ldvt = c->keys_pad;
+        a.out = c->B("encoder_attn"); a.ldo = 256; a.rows = 8 * S_e; a.keys = S_e; a.scale = 0.0625f;
+        a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = 0;
+        c->note(launch_mqa_attention(a, 4, s), "prefix attn");
+        gemm(c->B("encoder_attn"), 2048, S_e, S_e, c->TW("t_encoder_attn_o_w", i), nullptr, 2048, 2048, EPI_PARTIAL, GemmP{}, "prefix o");
+        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix o reduce");
+        GemmP g{}; g.out = c->B("encoder_hidden"); g.ldo = 16384;
+        gemm(c->B("encoder_x_norm"), 2048, S_e, S_e, c->TW("t_encoder_ffn_gate_w", i), c->TW("t_encoder_ffn_up_w", i), 2048, 16384, EPI_GEGLU, g, "prefix geglu");
+        gemm(c->B("encoder_hidden"), 16384, S_e, S_e, c->TW("t_encoder_ffn_down_w", i), nullptr, 16384, 2048, EPI_PARTIAL, GemmP{}, "prefix down");
+        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix down reduce");
+    }
+
+    void skinny(const bf16_t* A, int lda, int M, const bf16_t* B0, const bf16_t* B1, int K, int N, int norm, const bf16_t* style,
+                int epi, SkinnyP extra, const char* what) {
+        SkinnyP p = extra;
+        p.A = A; p.lda = lda; p.M = M; p.B0 = B0; p.B1 = B1; p.K = K; p.N16 = n16_tiles(N); p.K32p = k32_padded(K);
+        p.norm = norm; p.style = style; p.eps = 1e-6f;
+        c->note(launch_skinny(p, epi, s), what);
+    }
+
+    void suffix_init() {
+        if (pi05) return;
+        launch_small_linear(c->W("observation_state_normalized"), 32, c->W("decoder_state_in_proj_w"), c->W("decoder_state_in_proj_b"),
+                            c->B("decoder_state_buf"), 1024, 1, 32, 1024, 0, s);
+        c->note(0, "state proj");
+    }
+
+    void suffix_step_begin(int t) {
+        const int ch = d.chunk_size;
+        if (!pi05) {
+            launch_copy_rows(c->B("decoder_state_buf"), 1024, c->B("decoder_x"), 1024, 1, 1024, s); c->note(0, "state row");
+            launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_fused_in_proj_w"),
+                                c->W("decoder_action_fused_time_biases", 1024, t % 10), c->B("decoder_x_buf"), 1024, ch, 32, 1024, 1, s);
+            c->note(0, "action in");
+            SkinnyP e{}; e.out = c->B("decoder_x") + 1024; e.ldo = 1024; e.bias = c->W("decoder_action_mlp_b");
+            skinny(c->B("decoder_x_buf"), 1024, ch, c->TW("t_decoder_action_mlp_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS, e, "action mlp");
+        } else {
+            launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_in_proj_w"), c->W("decoder_action_in_proj_b"),
+                                c->B("decoder_x"), 1024, ch, 32, 1024, 0, s);
+            c->note(0, "action in");
+        }
+    }
+
+    void suffix_layer(int t, int i) {
+        const int S_d = c->S_d, S_e = c->S_e, L = d.llm_layers;
+        const int norm = pi05 ? SN_ADARMS : SN_RMS;
+        const bf16_t* st_attn = pi05 ? c->B("decoder_style_attn") + ((size_t)t * L + i) * 3072 : nullptr;
+        const bf16_t* st_ffn = pi05 ? c->B("decoder_style_ffn") + ((size_t)t * L + i) * 3072 : nullptr;
+        SkinnyP q{}; q.rope = c->W("decoder_rope_weights"); q.q = c->B("decoder_q_buf"); q.k = Kc(i); q.vt = Vt(i); q.ldvt = c->keys_pad; q.kv_row0 = S_e;
+        skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_attn_qkv_w", i), nullptr, 1024, 2560, norm, st_attn, SK_QKV_ROPE, q, "suffix qkv");
+        AttnP a{};
+        a.q = c->B("decoder_q_buf"); a.ldq = 256; a.k = Kc(i); a.ldk = 256; a.vt = Vt(i); a.ldvt = c->keys_pad;
+        a.out = c->B("decoder_attn"); a.ldo = 256; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
+        a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
+        c->note(launch_mqa_attention(a, 8, s), "suffix attn");
+        SkinnyP o{}; o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
+        skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
+        SkinnyP g{}; g.out = c->B("decoder_hidden"); g.ldo = 4096;
+        skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_ffn_gate_w", i), c->TW("t_decoder_ffn_up_w", i), 1024, 4096, norm, st_ffn, SK_GEGLU, g, "suffix geglu");
+        SkinnyP dn{}; dn.out = c->B("decoder_x"); dn.ldo = 1024; dn.gate = pi05 ? st_ffn + 2048 : nullptr;
+        skinny(c->B("decoder_hidden"), 4096, S_d, c->TW("t_decoder_ffn_down_w", i), nullptr, 4096, 1024, SN_NONE, nullptr, SK_RES, dn, "suffix down");
+    }
+
+    void suffix_step_end(int t) {
+        const int ch = d.chunk_size;
+        SkinnyP e{}; e.out = c->W("diffusion_noise"); e.ldo = 32;
+        if (!pi05) {
+            e.bias = c->W("decoder_action_fused_out_proj_b");
+            skinny(c->B("decoder_x") + 1024, 1024, ch, c->TW("t_decoder_out_proj_w"), nullptr, 1024, 32, SN_RMS, nullptr, SK_RES, e, "euler");
+        } else {
+            e.bias = c->B("decoder_out_proj_b_scaled");
+            skinny(c->B("decoder_x"), 1024, ch, c->TW("t_decoder_out_proj_w"), nullptr, 1024, 32, SN_ADARMS,
+                   c->B("decoder_style_final") + (size_t)t * 3072, SK_RES, e, "euler");
+        }
+    }
+
+    int stage(int st, int layer, int step) {
+        switch (st) {
+            case RTVLA_STAGE_VISION_EMBED: vision_embed(); break;
+            case RTVLA_STAGE_VISION_LAYER: if (layer < 0 || layer >= d.vision_layers) return RTVLA_ERR_ARG; vision_layer(layer); break;
+            case RTVLA_STAGE_PROJECT: project(); break;
+            case RTVLA_STAGE_PREFIX_LAYER: if (layer < 0 || layer >= d.llm_layers) return RTVLA_ERR_ARG; prefix_layer(layer); break;
+            case RTVLA_STAGE_SUFFIX_INIT: suffix_init(); break;
+            case RTVLA_STAGE_SUFFIX_STEP_BEGIN: if (step < 0 || step >= d.num_steps) return RTVLA_ERR_ARG; suffix_step_begin(step); break;
+            case RTVLA_STAGE_SUFFIX_LAYER:
+                if (layer < 0 || layer >= d.llm_layers || step < 0 || step >= d.num_steps) return RTVLA_ERR_ARG;
+                suffix_layer(step, layer); break;
+            case RTVLA_STAGE_SUFFIX_STEP_END: if (step < 0 || step >= d.num_steps) return RTVLA_ERR_ARG; suffix_step_end(step); break;
+            default: return RTVLA_ERR_ARG;
+        }
+        return 0;
+    }
+
+    void forward() {
+        vision_embed();
+        for (int i = 0; i < d.vision_layers; ++i) vision_layer(i);
+        project();
+        for (int i = 0; i < d.llm_layers; ++i) prefix_layer(i);
+        suffix_init();
+        for (int t = 0; t < d.num_steps; ++t) {
+            suffix_step_begin(t);
+            for (int i = 0; i < d.llm_layers; ++i) suffix_layer(t, i);
+            suffix_step_end(t);
+        }
+    }
+
+    // one-time device work
+    void prepare() {
+        const int V = d.vision_layers, L = d.llm_layers;
+        launch_fill_zero(c->ws + c->act_begin, c->ws_bytes - c->act_begin, s);
+        auto tile = [&](const char* src, const char* dst, int K, int N, int layers) {
+            for (int i = 0; i < layers; ++i) launch_pretile(c->W(src, (size_t)K * N, i), K, N, c->TW(dst, i), s);
+        };
+        tile("vision_patch_embedding_w", "t_vision_patch_embedding_w", 588, 1152, 1);
+        tile("vision_attn_qkv_w", "t_vision_attn_qkv_w", 1152, 3456, V);
+        tile("vision_attn_o_w", "t_vision_attn_o_w", 1152, 1152, V);
+        tile("vision_ffn_up_w", "t_vision_ffn_up_w", 1152, 4304, V);
+        tile("vision_ffn_down_w", "t_vision_ffn_down_w", 4304, 1152, V);
+        tile("encoder_multi_modal_projector_w", "t_encoder_multi_modal_projector_w", 1152, 2048, 1);
+        tile("encoder_attn_qkv_w", "t_encoder_attn_qkv_w", 2048, 2560, L);
+        tile("encoder_attn_o_w", "t_encoder_attn_o_w", 2048, 2048, L);
+        tile("encoder_ffn_gate_w", "t_encoder_ffn_gate_w", 2048, 16384, L);
+        tile("encoder_ffn_up_w", "t_encoder_ffn_up_w", 2048, 16384, L);
+        tile("encoder_ffn_down_w", "t_encoder_ffn_down_w", 16384, 2048, L);
+        tile("decoder_attn_qkv_w", "t_decoder_attn_qkv_w", 1024, 2560, L);
+        tile("decoder_attn_o_w", "t_decoder_attn_o_w", 2048, 1024, L);
+        tile("decoder_ffn_gate_w", "t_decoder_ffn_gate_w", 1024, 4096, L);
+        tile("decoder_ffn_up_w", "t_decoder_ffn_up_w", 1024, 4096, L);
+        tile("decoder_ffn_down_w", "t_decoder_ffn_down_w", 4096, 1024, L);
+        if (!pi05) {
+            tile("decoder_action_mlp_w", "t_decoder_action_mlp_w", 1024, 1024, 1);
+            tile("decoder_action_fused_out_proj_w", "t_decoder_out_proj_w", 1024, 32, 1);
+            return;
+        }
+        // Pi05: out-proj scaled by -1/num_steps (pi05_infer.py:669-671), then the time conditioning (:673-722)
+        const float dt = -1.0f / (float)d.num_steps;
+        launch_copy_bytes(c->W("decoder_action_out_proj_w"), c->B("decoder_out_proj_w_scaled"), 1024 * 32 * 2, s);
+        launch_scale_inplace(c->B("decoder_out_proj_w_scaled"), 1024 * 32, dt, s);
+        launch_copy_bytes(c->W("decoder_action_out_proj_b"), c->B("decoder_out_proj_b_scaled"), 64, s);
+        launch_scale_inplace(c->B("decoder_out_proj_b_scaled"), 32, dt, s);
+        launch_pretile(c->B("decoder_out_proj_w_scaled"), 1024, 32, c->TW("t_decoder_out_proj_w"), s);
+        tile("decoder_time_mlp_in_w", "t_decoder_time_mlp_in_w", 1024, 1024, 1);
+        tile("decoder_time_mlp_out_w", "t_decoder_time_mlp_out_w", 1024, 1024, 1);
+        tile("decoder_pre_attn_norm_mod_w", "t_decoder_pre_attn_norm_mod_w", 1024, 3072, L);
+        tile("decoder_pre_ffn_norm_mod_w", "t_decoder_pre_ffn_norm_mod_w", 1024, 3072, L);
+        tile("decoder_final_norm_mod_w", "t_decoder_final_norm_mod_w", 1024, 3072, 1);
+        const int T = d.num_steps;
+        SkinnyP e{}; e.out = c->B("decoder_x_buf"); e.ldo = 1024; e.bias = c->W("decoder_time_mlp_in_b");
+        skinny(c->W("decoder_time_embeds"), 1024, T, c->TW("t_decoder_time_mlp_in_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS_SILU, e, "time mlp in");
+        e.out = c->B("decoder_time_emb"); e.bias = c->W("decoder_time_mlp_out_b");
+        skinny(c->B("decoder_x_buf"), 1024, T, c->TW("t_decoder_time_mlp_out_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS_SILU, e, "time mlp out");
+        for (int i = 0; i < L; ++i) {
+            SkinnyP m{}; m.ldo = L * 3072;
+            m.out = c->B("decoder_style_attn") + (size_t)i * 3072; m.bias = c->W("decoder_pre_attn_norm_mod_b", 3072, i);
+            skinny(c->B("decoder_time_emb"), 1024, T, c->TW("t_decoder_pre_attn_norm_mod_w", i), nullptr, 1024, 3072, SN_NONE, nullptr, SK_BIAS, m, "style attn");
+            m.out = c->B("decoder_style_ffn") + (size_t)i * 3072; m.bias = c->W("decoder_pre_ffn_norm_mod_b", 3072, i);
+            skinny(c->B("decoder_time_emb"), 1024, T, c->TW("t_decoder_pre_ffn_norm_mod_w", i), nullptr, 1024, 3072, SN_NONE, nullptr, SK_BIAS, m, "style ffn");
+        }
+        SkinnyP f{}; f.ldo = 3072; f.out = c->B("decoder_style_final"); f.bias = c->W("decoder_final_norm_mod_b");
+        skinny(c->B("decoder_time_emb"), 1024, T, c->TW("t_decoder_final_norm_mod_w"), nullptr, 1024, 3072, SN_NONE, nullptr, SK_BIAS, f, "style final");
+    }
+};
+
+int check_ready(rtvla_ctx* c, bool need_prepared) {
+    if (!c) return RTVLA_ERR_ARG;
+    if (!c->ws) return c->fail(RTVLA_ERR_STATE, "workspace not bound");
+    for (auto& t : c->tensors)
+        if (t.required && !t.bound) return c->fail(RTVLA_ERR_UNBOUND, "tensor not bound: " + t.name);
+    if (need_prepared && !c->prepared) return c->fail(RTVLA_ERR_STATE, "rtvla_prepare has not run");
+    return 0;
+}
+
+int hip_fail(rtvla_ctx* c, hipError_t e, const char* what) {
+    return c->fail(RTVLA_ERR_DEVICE, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+}  // namespace
+
+extern "C" {
+
+int rtvla_version(void) { return 1; }
+
+int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out) {
+    if (!dims || !out) return RTVLA_ERR_ARG;
+    *out = nullptr;
+    const rtvla_dims& d = *dims;
+    if (d.model != RTVLA_PI0 && d.model != RTVLA_PI05) return RTVLA_ERR_ARG;
+    if (d.num_views < 1 || d.num_views > 4 || d.prompt_len < 0 || d.chunk_size < 1 || d.num_steps < 1) return RTVLA_ERR_ARG;
+    if (d.vision_layers < 1 || d.llm_layers < 1) return RTVLA_ERR_ARG;
+    const int S_d = d.chunk_size + (d.model == RTVLA_PI0 ? 1 : 0);
+    if (S_d > 64) return RTVLA_ERR_LIMIT;
+    if (d.model == RTVLA_PI05 && d.num_steps > 10) return RTVLA_ERR_LIMIT;      // decoder_time_embeds has 10 rows
+    if (d.prompt_len > 4096) return RTVLA_ERR_LIMIT;
+    rtvla_ctx* c = new (std::nothrow) rtvla_ctx();
+    if (!c) return RTVLA_ERR_ARG;
+    c->d = d;
+    c->S_v = 256 * d.num_views;
+    c->S_e = c->S_v + d.prompt_len;
+    c->S_d = S_d;
+    c->keys = c->S_e + c->S_d;
+    c->keys_pad = ((c->keys + 63) / 64) * 64;
+    build_tables(c);
+    *out = c;
+    return RTVLA_OK;
+}
+
+int rtvla_destroy(rtvla_ctx* c) {
+    if (!c) return RTVLA_ERR_ARG;
+    if (c->exec) hipGraphExecDestroy(c->exec);
+    if (c->graph) hipGraphDestroy(c->graph);
+    delete c;
+    return RTVLA_OK;
+}
+
+const char* rtvla_last_error(const rtvla_ctx* c) { return c ? c->err.c_str() : "null context"; }
+
+int rtvla_tensor_count(const rtvla_ctx* c) { return c ? (int)c->tensors.size() : 0; }
+
+int rtvla_tensor_info(const rtvla_ctx* c, int index, const char** name, int32_t* elem_bytes, int32_t* rank,
+                      int64_t shape[4], int32_t* is_weight, int32_t* required) {
+    if (!c || index < 0 || index >= (int)c->tensors.size()) return RTVLA_ERR_ARG;
+    const Tensor& t = c->tensors[index];
+    if (name) *name = t.name.c_str();
+    if (elem_bytes) *elem_bytes = t.elem;
+    if (rank) *rank = t.rank;
+    if (shape) for (int i = 0; i < 4; ++i) shape[i] = t.shape[i];
+    if (is_weight) *is_weight = t.weight;
+    if (required) *required = t.required;
+    return RTVLA_OK;
+}
+
+int rtvla_bind(rtvla_ctx* c, const char* name, void* ptr, size_t bytes) {
+    if (!c || !name) return RTVLA_ERR_ARG;
+    auto it = c->tindex.find(name);
+    if (it == c->tindex.end()) return c->fail(RTVLA_ERR_NAME, std::string("unknown tensor: ") + name);
+    Tensor& t = c->tensors[it->second];
+    if (bytes != t.bytes()) return c->fail(RTVLA_ERR_SIZE, std::string("size mismatch for ") + name + ": got " + std::to_string(bytes) + ", want " + std::to_string(t.bytes()));
+    if (!ptr && bytes) return c->fail(RTVLA_ERR_ARG, std::string("null pointer for ") + name);
+    if (((uintptr_t)ptr & 15) != 0) return c->fail(RTVLA_ERR_ARG, std::string("pointer not 16-byte aligned: ") + name);
+    t.ptr = ptr; t.bound = true;
+    c->prepared = false;
+    return RTVLA_OK;
+}
+
+size_t rtvla_workspace_bytes(const rtvla_ctx* c) { return c ? c->ws_bytes : 0; }
+
+int rtvla_bind_workspace(rtvla_ctx* c, void* ptr, size_t bytes) {
+    if (!c || !ptr) return RTVLA_ERR_ARG;
+    if (bytes < c->ws_bytes) return c->fail(RTVLA_ERR_SIZE, "workspace too small");
+    if (((uintptr_t)ptr & 255) != 0) return c->fail(RTVLA_ERR_ARG, "workspace not 256-byte aligned");
+    c->ws = (char*)ptr; c->prepared = false;
+    return RTVLA_OK;
+}
+
+int rtvla_buffer_count(const rtvla_ctx* c) { return c ? (int)c->bufs.size() : 0; }
+
+int rtvla_buffer_info(const rtvla_ctx* c, int index, const char** name, size_t* offset, int64_t* rows, int64_t* cols,
+                      int64_t* ld, int32_t* elem_bytes) {
+    if (!c || index < 0 || index >= (int)c->bufs.size()) return RTVLA_ERR_ARG;
+    const WsBuf& b = c->bufs[index];
+    if (name) *name = b.name.c_str();
+    if (offset) *offset = b.offset;
+    if (rows) *rows = b.rows;
+    if (cols) *cols = b.cols;
+    if (ld) *ld = b.ld;
+    if (elem_bytes) *elem_bytes = b.elem;
+    return RTVLA_OK;
+}
+
+int rtvla_prepare(rtvla_ctx* c, void* stream) {
+    if (int rc = check_ready(c, false)) return rc;
+    c->status = 0; c->launches = 0;
+    Sched(c, (hipStream_t)stream).prepare();
+    if (c->status) return c->status;
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(c, e, "prepare");
+    c->prepared = true;
+    return RTVLA_OK;
+}
+
+int rtvla_forward(rtvla_ctx* c, void* stream) {
+    if (int rc = check_ready(c, true)) return rc;
+    c->status = 0; c->launches = 0;
+    Sched(c, (hipStream_t)stream).forward();
+    return c->status;
+}
+
+int rtvla_forward_stage(rtvla_ctx* c, int stage, int layer, int step, void* stream) {
+    if (int rc = check_ready(c, true)) return rc;
+    c->status = 0; c->launches = 0;
+    int rc = Sched(c, (hipStream_t)stream).stage(stage, layer, step);
+    if (rc) return c->fail(rc, "bad stage / layer / step");
+    return c->status;
+}
+
+int rtvla_graph_capture(rtvla_ctx* c, void* stream) {
+    if (int rc = check_ready(c, true)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    // one eager run first: sets per-kernel attributes outside the capture and surfaces launch errors
+    if (int rc = rtvla_forward(c, stream)) return rc;
+    hipError_t e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(c, e, "eager forward before capture");
+    if (c->exec) { hipGraphExecDestroy(c->exec); c->exec = nullptr; }
+    if (c->graph) { hipGraphDestroy(c->graph); c->graph = nullptr; }
+    e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return hip_fail(c, e, "hipStreamBeginCapture");
+    c->status = 0; c->launches = 0;
+    Sched(c, s).forward();
+    e = hipStreamEndCapture(s, &c->graph);
+    if (e != hipSuccess) return hip_fail(c, e, "hipStreamEndCapture");
+    if (c->status) return c->status;
+    e = hipGraphInstantiate(&c->exec, c->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) return hip_fail(c, e, "hipGraphInstantiate");
+    return RTVLA_OK;
+}
+
+int rtvla_graph_launch(rtvla_ctx* c, void* stream) {
+    if (!c) return RTVLA_ERR_ARG;
+    if (!c->exec) return c->fail(RTVLA_ERR_STATE, "no graph captured");
+    hipError_t e = hipGraphLaunch(c->exec, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(c, e, "hipGraphLaunch");
+    return RTVLA_OK;
+}
+
+int rtvla_launch_count(const rtvla_ctx* c) { return c ? c->launches : 0; }
+
+int rtvla_time_stage(rtvla_ctx* c, int stage, int layer, int step, int iters, void* stream, float* mean_ms) {
+    if (int rc = check_ready(c, true)) return rc;
+    if (iters < 1 || !mean_ms) return RTVLA_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    hipEvent_t a, b;
+    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
+    Sched sc(c, s);
+    c->status = 0;
+    int rc = sc.stage(stage, layer, step);      // warm-up
+    if (!rc) {
+        hipEventRecord(a, s);
+        for (int i = 0; i < iters && !rc; ++i) rc = sc.stage(stage, layer, step);
+        hipEventRecord(b, s);
+        hipError_t e = hipEventSynchronize(b);
+        if (e != hipSuccess) rc = hip_fail(c, e, "time_stage");
+        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / iters; }
+    }
+    hipEventDestroy(a); hipEventDestroy(b);
+    if (rc) return rc;
+    return c->status;
+}
+
+int rtvla_time_forward(rtvla_ctx* c, int iters, void* stream, float* ms_out) {
+    if (int rc = check_ready(c, true)) return rc;
+    if (iters < 1 || !ms_out) return RTVLA_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    hipEvent_t a, b;
+    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
+    int rc = 0;
+    for (int i = 0; i < iters && !rc; ++i) {
+        hipEventRecord(a, s);
+        rc = c->exec ? rtvla_graph_launch(c, stream) : rtvla_forward(c, stream);
+        hipEventRecord(b, s);
+        hipError_t e = hipEventSynchronize(b);
+        if (e != hipSuccess) rc = hip_fail(c, e, "time_forward");
+        else hipEventElapsedTime(&ms_out[i], a, b);
+    }
+    hipEventDestroy(a); hipEventDestroy(b);
+    return rc;
+}
+
+size_t rtvla_pretile_elems(int K, int N) { return (K > 0 && N > 0) ? tiled_elems(K, N) : 0; }
+
+int rtvla_pretile(const void* w, int K, int N, void* w_tiled, void* stream) {
+    if (!w || !w_tiled || K <= 0 || N <= 0) return RTVLA_ERR_ARG;
+    launch_pretile((const bf16_t*)w, K, N, (bf16_t*)w_tiled, (hipStream_t)stream);
+    return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
+}
+
+}  // extern "C"

@@ -1,0 +1,215 @@
+// Weight-streaming GEMM for the action expert (M <= 64 rows), replacing the decoder-side Triton
+// kernels of /root/reference/pi0_infer.py:82-124, :693-725, :939-1039, :1122-1163 and
+// /root/reference/pi05_infer.py:22-64, :78-113, :127-195.
+//
+// One workgroup owns one 16-column tile of the output and all of K; its 8 waves split K.  Each wave
+// issues all of its weight-fragment loads up front (coalesced 1 KB reads of the pre-tiled layout,
+// straight into registers), reads its slice of the activations in MFMA operand order from L2,
+// multiplies, and the waves reduce through LDS.  Because the workgroup sees every activation row
+// over all of K, the RMS / adaRMS normalisation that precedes the GEMM in the reference is computed
+// here from the same registers (wavefront reduction, no separate launch), and the epilogue applies
+// RoPE + KV-cache append, GeGLU, residual (+gate) or the Euler update in place.
+#include "kernels.h"
+
+namespace {
+
+constexpr int SK_WAVES = 8;
+constexpr int SK_MTS = 4;      // 4 x 16 = 64 rows
+constexpr int SK_CH = 4;       // k32 blocks per A-prefetch chunk
+
+template <int NCH, int NORM, int EPI>
+__global__ __launch_bounds__(SK_WAVES * 64)
+void skinny_kernel(SkinnyP p) {
+    constexpr int KBW = NCH * SK_CH;
+    constexpr bool DUAL = (EPI == SK_GEGLU);
+    constexpr int NB = DUAL ? 2 : 1;
+    static_assert(NORM == SN_NONE || NCH == 1, "the fused norm needs the whole K slice in registers");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    f32x4* red = (f32x4*)smem_raw;                                        // [WAVES][NB*MTS][64]
+    float* ssq = (float*)(smem_raw + (size_t)SK_WAVES * NB * SK_MTS * 64 * 16);   // [WAVES][64]
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int g = lane >> 4, r = lane & 15;
+    const int tile = blockIdx.x;
+    const int kb0 = w * KBW;
+
+    // ---- weight fragments: the HBM stream, all in flight at once ----
+    bf16x8 b[NB][KBW];
+    {
+        const bf16_t* bp0 = p.B0 + ((size_t)tile * p.K32p + kb0) * 512 + lane * 8;
+#pragma unroll
+        for (int i = 0; i < KBW; ++i) b[0][i] = *(const bf16x8*)(bp0 + (size_t)i * 512);
+        if constexpr (DUAL) {
+            const bf16_t* bp1 = p.B1 + ((size_t)tile * p.K32p + kb0) * 512 + lane * 8;
+#pragma unroll
+            for (int i = 0; i < KBW; ++i) b[1][i] = *(const bf16x8*)(bp1 + (size_t)i * 512);
+        }
+    }
+    const bf16_t* arow[SK_MTS];
+#pragma unroll
+    for (int mt = 0; mt < SK_MTS; ++mt) {
+        const int row = min(mt * 16 + r, p.M - 1);
+        arow[mt] = p.A + (size_t)row * p.lda + kb0 * 32 + 8 * g;
+    }
+    f32x4 acc[NB][SK_MTS];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mt = 0; mt < SK_MTS; ++mt) acc[nb][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    bf16x8 a[2][SK_MTS][SK_CH];
+    auto load_a = [&](int c, bf16x8 (&dst)[SK_MTS][SK_CH]) {
+#pragma unroll
+        for (int mt = 0; mt < SK_MTS; ++mt)
+#pragma unroll
+            for (int i = 0; i < SK_CH; ++i) dst[mt][i] = *(const bf16x8*)(arow[mt] + (c * SK_CH + i) * 32);
+    };
+    load_a(0, a[0]);
+
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        if (c + 1 < NCH) load_a(c + 1, a[(c + 1) & 1]);
+        if constexpr (NORM != SN_NONE) {
+            // row sums of squares over this wave's K slice, then over the 8 waves
+            float ss[SK_MTS];
+#pragma unroll
+            for (int mt = 0; mt < SK_MTS; ++mt) {
+                float s = 0.f;
+#pragma unroll
+                for (int i = 0; i < SK_CH; ++i)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) { const float x = bf2f(a[0][mt][i][j]); s += x * x; }
+                s += __shfl_xor(s, 16, 64);
+                s += __shfl_xor(s, 32, 64);
+                ss[mt] = s;
+            }
+            if (g == 0) {
+#pragma unroll
+                for (int mt = 0; mt < SK_MTS; ++mt) ssq[w * 64 + mt * 16 + r] = ss[mt];
+            }
+            __syncthreads();
+            float f[SK_MTS];
+#pragma unroll
+            for (int mt = 0; mt < SK_MTS; ++mt) {
+                float t = 0.f;
+#pragma unroll
+                for (int ww = 0; ww < SK_WAVES; ++ww) t += ssq[ww * 64 + mt * 16 + r];
+                f[mt] = rsqrtf(t / (float)p.K + p.eps);
+                if (NORM == SN_RMS) f[mt] = round_bf16(f[mt]);      // the reference keeps the factor in bf16
+            }
+#pragma unroll
+            for (int i = 0; i < SK_CH; ++i) {
+                bf16x8 sc, sh;
+                if constexpr (NORM == SN_ADARMS) {
+                    sc = *(const bf16x8*)(p.style + (kb0 + i) * 32 + 8 * g);
+                    sh = *(const bf16x8*)(p.style + p.K + (kb0 + i) * 32 + 8 * g);
+                }
+#pragma unroll
+                for (int mt = 0; mt < SK_MTS; ++mt)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        float x = bf2f(a[0][mt][i][j]) * f[mt];
+                        if constexpr (NORM == SN_ADARMS) x = x * (1.0f + bf2f(sc[j])) + bf2f(sh[j]);
+                        a[0][mt][i][j] = f2bf(x);
+                    }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < SK_CH; ++i)
+#pragma unroll
+            for (int mt = 0; mt < SK_MTS; ++mt)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    acc[nb][mt] = mfma16(b[nb][c * SK_CH + i], a[c & 1][mt][i], acc[nb][mt]);
+    }
+
+    // ---- reduce the 8 K-slices through LDS; wave mt finishes row tile mt ----
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mt = 0; mt < SK_MTS; ++mt) red[((size_t)w * NB * SK_MTS + nb * SK_MTS + mt) * 64 + lane] = acc[nb][mt];
+    __syncthreads();
+    if (w >= SK_MTS) return;
+    const int mt = w;
+    const int m = mt * 16 + r;
+    f32x4 v[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ww = 0; ww < SK_WAVES; ++ww) t += red[((size_t)ww * NB * SK_MTS + nb * SK_MTS + mt) * 64 + lane];
+        v[nb] = t;
+    }
+    if (m >= p.M) return;
+    const int n0 = tile * 16 + 4 * g;
+    if constexpr (EPI == SK_BIAS || EPI == SK_BIAS_SILU) {
+        f32x4 o = v[0];
+        const bf16x4 bb = load4(p.bias + n0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { o[e] += bf2f(bb[e]); if (EPI == SK_BIAS_SILU) o[e] = siluf(o[e]); }
+        store4(p.out + (size_t)m * p.ldo + n0, pack4(o));
+    } else if constexpr (EPI == SK_RES) {
+        f32x4 o = v[0];
+        if (p.gate) { const bf16x4 gg = load4(p.gate + n0); for (int e = 0; e < 4; ++e) o[e] *= bf2f(gg[e]); }
+        if (p.bias) { const bf16x4 bb = load4(p.bias + n0); for (int e = 0; e < 4; ++e) o[e] += bf2f(bb[e]); }
+        const bf16x4 old = load4(p.out + (size_t)m * p.ldo + n0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] += bf2f(old[e]);
+        store4(p.out + (size_t)m * p.ldo + n0, pack4(o));
+    } else if constexpr (EPI == SK_GEGLU) {
+        store4(p.out + (size_t)m * p.ldo + n0,
+               pack4(gelu_tanh(v[0][0]) * v[1][0], gelu_tanh(v[0][1]) * v[1][1], gelu_tanh(v[0][2]) * v[1][2], gelu_tanh(v[0][3]) * v[1][3]));
+    } else if constexpr (EPI == SK_QKV_ROPE) {
+        f32x4 o = v[0];
+        if (n0 < 2304) {
+            const bf16x4 cs = load4(p.rope + (size_t)m * 256 + (n0 & 255));
+            const float c0 = bf2f(cs[0]), s0 = bf2f(cs[1]), c1 = bf2f(cs[2]), s1 = bf2f(cs[3]);
+            const f32x4 x = o;
+            o[0] = x[0] * c0 - x[1] * s0; o[1] = x[1] * c0 + x[0] * s0;
+            o[2] = x[2] * c1 - x[3] * s1; o[3] = x[3] * c1 + x[2] * s1;
+            if (n0 < 2048) store4(p.q + (size_t)m * 2048 + n0, pack4(o));
+            else store4(p.k + (size_t)(p.kv_row0 + m) * 256 + (n0 - 2048), pack4(o));
+        } else {
+            const int d = n0 - 2304;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) p.vt[(size_t)(d + e) * p.ldvt + p.kv_row0 + m] = f2bf(o[e]);
+        }
+    }
+}
+
+template <int NCH, int NORM, int EPI>
+int launch_inst(const SkinnyP& p, hipStream_t s) {
+    constexpr int NB = (EPI == SK_GEGLU) ? 2 : 1;
+    const size_t smem = (size_t)SK_WAVES * NB * SK_MTS * 64 * 16 + (size_t)SK_WAVES * 64 * 4;
+    auto kern = skinny_kernel<NCH, NORM, EPI>;
+    if (smem > 65536) {
+        static bool done = false;
+        if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
+    }
+    hipLaunchKernelGGL(kern, dim3(p.N16), dim3(SK_WAVES * 64), smem, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+}
+
+}  // namespace
+
+int launch_skinny(const SkinnyP& p, int epi, hipStream_t s) {
+    if (p.M <= 0 || p.M > 64 || p.N16 <= 0) return 1;
+    if (p.K != 1024 && p.K != 2048 && p.K != 4096) return 1;
+    if (p.K32p < p.K / 32 || p.lda < p.K) return 1;
+    const int nch = p.K / (32 * SK_WAVES * SK_CH);
+    if (p.norm != SN_NONE && nch != 1) return 1;
+    if (p.norm == SN_ADARMS && !p.style) return 1;
+#define SK_CASE(NCH_, NORM_, EPI_) if (nch == NCH_ && p.norm == NORM_ && epi == EPI_) return launch_inst<NCH_, NORM_, EPI_>(p, s)
+    SK_CASE(1, SN_RMS, SK_QKV_ROPE);
+    SK_CASE(1, SN_ADARMS, SK_QKV_ROPE);
+    SK_CASE(1, SN_RMS, SK_GEGLU);
+    SK_CASE(1, SN_ADARMS, SK_GEGLU);
+    SK_CASE(1, SN_NONE, SK_BIAS);
+    SK_CASE(1, SN_NONE, SK_BIAS_SILU);
+    SK_CASE(1, SN_RMS, SK_RES);
+    SK_CASE(1, SN_ADARMS, SK_RES);
+    SK_CASE(2, SN_NONE, SK_RES);
+    SK_CASE(4, SN_NONE, SK_RES);
+#undef SK_CASE
+    return 2;
+}
