@@ -134,6 +134,13 @@ int rtvla_launch_count(const rtvla_ctx* ctx);
  * per run.  Synchronises the stream. */
 int rtvla_time_stage(rtvla_ctx* ctx, int stage, int layer, int step, int iters, void* hip_stream, float* mean_ms);
 
+/* Measurement helper (no reference counterpart): as rtvla_time_stage, but enqueue only the
+ * `launch_index`-th kernel launch of the stage (0-based, in schedule order), so that one kernel's
+ * mean duration is measured live with HIP events on the stream it is launched on.  The launch's
+ * name is copied to name_out.  Returns RTVLA_ERR_ARG when the stage has fewer launches. */
+int rtvla_time_launch(rtvla_ctx* ctx, int stage, int layer, int step, int launch_index, int iters, void* hip_stream,
+                      float* mean_ms, char* name_out, size_t name_cap);
+
 /* Measurement helper: time `iters` graph replays (or eager forwards when no graph is captured)
  * individually with HIP events on the stream; writes per-iteration milliseconds to ms_out[iters]. */
 int rtvla_time_forward(rtvla_ctx* ctx, int iters, void* hip_stream, float* ms_out);

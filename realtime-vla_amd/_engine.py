@@ -75,3 +75,25 @@ class Engine:
 
     def run_eager(self):
         self.ctx.forward(torch.cuda.current_stream(self.device).cuda_stream)
+
+
+# ---- layout helpers for the library's fragment-tiled activations (taps, tests) -------------------
+def untile_ft(flat, rows, cols):
+    """Row-major copy of a fragment-tiled [rows][cols] matrix (rows % 16 == 0, cols % 32 == 0):
+    tile (row/16, col/32) holds 64 lanes x 8 elements, lane = row%16 + 16*((col%32)/8)."""
+    t = flat.reshape(-1)[: rows * cols].view(rows // 16, cols // 32, 4, 16, 8)
+    return t.permute(0, 3, 1, 2, 4).reshape(rows, cols)
+
+
+def tile_ft(mat):
+    """Inverse of untile_ft."""
+    rows, cols = mat.shape
+    t = mat.reshape(rows // 16, 16, cols // 32, 4, 8)
+    return t.permute(0, 2, 3, 1, 4).reshape(-1)
+
+
+def untile_vt(flat, d, keys_pad):
+    """Row-major [d][keys_pad] copy of the transposed-V layout: tile (d/16, key/32), lane = d%16 + 16 g,
+    register j holding key 32*tile + 4 g + (j & 3) + 16 (j >> 2)."""
+    t = flat.reshape(-1)[: d * keys_pad].view(d // 16, keys_pad // 32, 4, 16, 2, 4)     # [dt][kt][g][r][hi][lo]
+    return t.permute(0, 3, 1, 4, 2, 5).reshape(d, keys_pad)

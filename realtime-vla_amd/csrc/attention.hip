@@ -24,8 +24,8 @@ RTVLA_DEVICE bf16x8 cat44(bf16x4 lo, bf16x4 hi) {
     return v;
 }
 
-template <int WAVES, int MQ>
-__global__ __launch_bounds__(WAVES * 64)
+template <int WAVES, int MQ, int NTK>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void mqa_kernel(AttnP p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     f32x4* obuf = (f32x4*)smem_raw;                                   // [WAVES][16][64]
@@ -42,10 +42,10 @@ void mqa_kernel(AttnP p) {
     bf16x8 qf[MQ][8];
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
-        const int row = min(m0 + mq * 16 + r, p.rows - 1);
-        const bf16_t* qp = p.q + (size_t)row * p.ldq + 8 * g;
+        // fragment-tiled Q: one contiguous 1 KB read per fragment (row tiles past the end are padding)
+        const bf16_t* qp = p.q + ((size_t)(blockIdx.x * MQ + mq) * 8 * 64 + lane) * 8;
 #pragma unroll
-        for (int kd = 0; kd < 8; ++kd) qf[mq][kd] = *(const bf16x8*)(qp + kd * 32);
+        for (int kd = 0; kd < 8; ++kd) qf[mq][kd] = *(const bf16x8*)(qp + kd * 512);
     }
     f32x4 o[MQ][16];
     float mrun[MQ], lrun[MQ];
@@ -56,33 +56,55 @@ void mqa_kernel(AttnP p) {
         for (int dt = 0; dt < 16; ++dt) o[mq][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    const int nkb = (p.keys + 63) >> 6;
+    constexpr int KBS = NTK * 16;                    // keys per block
+    const int nkb = (p.keys + KBS - 1) / KBS;
+    const int keys32 = p.ldvt >> 5;
+    bf16x8 kf[NTK][8];        // K fragments of one key block (A operand of S^T = K Q^T)
+    bf16x8 vf[16][NTK / 2];      // V^T fragments of the block, in the key order the P registers have
+    auto load_k = [&](int kb) {
+#pragma unroll
+        for (int nt = 0; nt < NTK; ++nt) {
+            const bf16_t* kp = p.k + ((size_t)(kb * NTK + nt) * 8 * 64 + lane) * 8;
+#pragma unroll
+            for (int kd = 0; kd < 8; ++kd) kf[nt][kd] = *(const bf16x8*)(kp + kd * 512);
+        }
+    };
+    auto load_v = [&](int kb) {
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) {
+            const bf16_t* vp = p.vt + ((size_t)(dt * keys32 + kb * (NTK / 2)) * 64 + lane) * 8;
+#pragma unroll
+            for (int kk = 0; kk < NTK / 2; ++kk) vf[dt][kk] = *(const bf16x8*)(vp + kk * 512);
+        }
+    };
+    if (w < nkb) { load_k(w); load_v(w); }
+    __builtin_amdgcn_sched_barrier(0);
+
     for (int kb = w; kb < nkb; kb += WAVES) {
-        const int key0 = kb * 64;
-        f32x4 st[MQ][4];
+        const int key0 = kb * KBS;
+        const int kb_next = min(kb + WAVES, nkb - 1);       // the last round re-reads a block instead of branching
+        f32x4 st[MQ][NTK];
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt) st[mq][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int nt = 0; nt < NTK; ++nt) st[mq][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) {
-            const int key = min(key0 + nt * 16 + r, p.keys - 1);
-            const bf16_t* kp = p.k + (size_t)key * p.ldk + 8 * g;
+        for (int nt = 0; nt < NTK; ++nt)
 #pragma unroll
-            for (int kd = 0; kd < 8; ++kd) {
-                const bf16x8 kf = *(const bf16x8*)(kp + kd * 32);
+            for (int kd = 0; kd < 8; ++kd)
 #pragma unroll
-                for (int mq = 0; mq < MQ; ++mq) st[mq][nt] = mfma16(kf, qf[mq][kd], st[mq][nt]);
-            }
-        }
-        bf16x8 pb[MQ][2];
+                for (int mq = 0; mq < MQ; ++mq) st[mq][nt] = mfma16(kf[nt][kd], qf[mq][kd], st[mq][nt]);
+        __builtin_amdgcn_sched_barrier(0);
+        load_k(kb_next);                                     // next block's K flies during softmax and P V
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 pb[MQ][NTK / 2];
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq) {
             const int row = m0 + mq * 16 + r;
             float mx = NEG_BIG;
-            bool vis[4][4];
+            bool vis[NTK][4];
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt)
+            for (int nt = 0; nt < NTK; ++nt)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const int key = key0 + nt * 16 + 4 * g + v;
@@ -100,7 +122,7 @@ void mqa_kernel(AttnP p) {
             const float alpha = __expf(mrun[mq] - mnew);
             float sum = 0.f;
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt)
+            for (int nt = 0; nt < NTK; ++nt)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const float e = vis[nt][v] ? __expf(st[mq][nt][v] - mnew) : 0.f;
@@ -114,18 +136,18 @@ void mqa_kernel(AttnP p) {
 #pragma unroll
             for (int dt = 0; dt < 16; ++dt) o[mq][dt] *= alpha;
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) pb[mq][kk] = cat44(pack4(st[mq][2 * kk]), pack4(st[mq][2 * kk + 1]));
+            for (int kk = 0; kk < NTK / 2; ++kk) pb[mq][kk] = cat44(pack4(st[mq][2 * kk]), pack4(st[mq][2 * kk + 1]));
         }
 #pragma unroll
-        for (int dt = 0; dt < 16; ++dt) {
-            const bf16_t* vp = p.vt + (size_t)(dt * 16 + r) * p.ldvt + key0 + 4 * g;
+        for (int dt = 0; dt < 16; ++dt)
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-                const bf16x8 vf = cat44(load4(vp + kk * 32), load4(vp + kk * 32 + 16));
+            for (int kk = 0; kk < NTK / 2; ++kk) {
 #pragma unroll
-                for (int mq = 0; mq < MQ; ++mq) o[mq][dt] = mfma16(vf, pb[mq][kk], o[mq][dt]);
+                for (int mq = 0; mq < MQ; ++mq) o[mq][dt] = mfma16(vf[dt][kk], pb[mq][kk], o[mq][dt]);
             }
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_v(kb_next);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- merge the key splits of the WAVES waves ----
@@ -160,47 +182,61 @@ void mqa_kernel(AttnP p) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ww = 0; ww < WAVES; ++ww) t += obuf[((size_t)ww * 16 + dt) * 64 + lane];
-            if (row < p.rows) store4(p.out + (size_t)row * p.ldo + dt * 16 + 4 * g, pack4(t * inv));
+            if (row < p.rows) {
+                const int d = dt * 16 + 4 * g;
+                // tiled output: the [tokens][8*256] matrix the suffix O-projection reads as MFMA fragments
+                bf16_t* dst = p.out_tiled ? p.out + ft_index(row >> 3, (row & 7) * 256 + d, 64) : p.out + (size_t)row * p.ldo + d;
+                store4(dst, pack4(t * inv));
+            }
         }
     }
 }
 
-// SigLIP: qk [views*256][2304] = Q(16 x 72) | K(16 x 72), vt [views*16][80][256], out [views*256][1152].
+// SigLIP: per (view, head) Q and K are fragment-tiled [256 tokens][96] (head dim 72 zero padded),
+// V^T is [80][256] in the permuted-key tile layout; out is row-major [views*256][1152].
 // One wave per 16 query rows over all 256 keys; 4 waves per workgroup.
-__global__ __launch_bounds__(256)
-void vision_attn_kernel(const bf16_t* __restrict__ qk, const bf16_t* __restrict__ vt, bf16_t* __restrict__ out) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ vt,
+                        bf16_t* __restrict__ out) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
     const int blk = blockIdx.x;                  // (view*16 + head)*4 + quarter
     const int quarter = blk & 3, vh = blk >> 2, head = vh & 15, view = vh >> 4;
-    const int row = view * 256 + quarter * 64 + w * 16 + r;       // query token (global row)
+    const int mtile = quarter * 4 + w;                             // 16-row tile of this wave inside the view
+    const int row = view * 256 + mtile * 16 + r;                   // query token (global row)
     const float scale = 0.11785113019775792f;                      // 1 / sqrt(72)
-    const bf16x8 zero8 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
+    const bf16_t* qb = q + (size_t)vh * (256 * 96) + lane * 8;
+    const bf16_t* kb_ = k + (size_t)vh * (256 * 96) + lane * 8;
+    const bf16_t* vb = vt + (size_t)vh * (80 * 256) + lane * 8;
     bf16x8 qf[3];
-    {
-        const bf16_t* qp = qk + (size_t)row * 2304 + head * 72 + 8 * g;
-        qf[0] = *(const bf16x8*)qp;
-        qf[1] = *(const bf16x8*)(qp + 32);
-        qf[2] = (g == 0) ? *(const bf16x8*)(qp + 64) : zero8;
-    }
+#pragma unroll
+    for (int kd = 0; kd < 3; ++kd) qf[kd] = *(const bf16x8*)(qb + (size_t)(mtile * 3 + kd) * 512);
+    // all K and V^T fragments of the 256 keys are requested up front (88 x 1 KB loads per wave)
+    bf16x8 kf[16][3];
+    bf16x8 vf[5][8];
+#pragma unroll
+    for (int nt = 0; nt < 16; ++nt)
+#pragma unroll
+        for (int kd = 0; kd < 3; ++kd) kf[nt][kd] = *(const bf16x8*)(kb_ + (size_t)(nt * 3 + kd) * 512);
+#pragma unroll
+    for (int dt = 0; dt < 5; ++dt)
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) vf[dt][kk] = *(const bf16x8*)(vb + (size_t)(dt * 8 + kk) * 512);
+    __builtin_amdgcn_sched_barrier(0);
+
     f32x4 o[5];
 #pragma unroll
     for (int dt = 0; dt < 5; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     float mrun = NEG_BIG, lrun = 0.f;
-    const bf16_t* vbase = vt + (size_t)vh * 80 * 256;
-
+#pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
-        const int key0 = kb * 64;
         f32x4 st[4];
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt) {
             st[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-            const bf16_t* kp = qk + (size_t)(view * 256 + key0 + nt * 16 + r) * 2304 + 1152 + head * 72 + 8 * g;
-            st[nt] = mfma16(*(const bf16x8*)kp, qf[0], st[nt]);
-            st[nt] = mfma16(*(const bf16x8*)(kp + 32), qf[1], st[nt]);
-            const bf16x8 k2 = (g == 0) ? *(const bf16x8*)(kp + 64) : zero8;
-            st[nt] = mfma16(k2, qf[2], st[nt]);
+#pragma unroll
+            for (int kd = 0; kd < 3; ++kd) st[nt] = mfma16(kf[kb * 4 + nt][kd], qf[kd], st[nt]);
         }
         float mx = NEG_BIG;
 #pragma unroll
@@ -226,10 +262,8 @@ void vision_attn_kernel(const bf16_t* __restrict__ qk, const bf16_t* __restrict_
 #pragma unroll
         for (int dt = 0; dt < 5; ++dt) {
             o[dt] *= alpha;
-            const bf16_t* vp = vbase + (size_t)(dt * 16 + r) * 256 + key0 + 4 * g;
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
-                o[dt] = mfma16(cat44(load4(vp + kk * 32), load4(vp + kk * 32 + 16)), pb[kk], o[dt]);
+            for (int kk = 0; kk < 2; ++kk) o[dt] = mfma16(vf[dt][kb * 2 + kk], pb[kk], o[dt]);
         }
     }
     const float inv = 1.0f / lrun;
@@ -240,10 +274,10 @@ void vision_attn_kernel(const bf16_t* __restrict__ qk, const bf16_t* __restrict_
     }
 }
 
-template <int WAVES, int MQ>
+template <int WAVES, int MQ, int NTK>
 int launch_mqa_inst(const AttnP& p, hipStream_t s) {
     const size_t smem = (size_t)WAVES * 16 * 64 * 16 + (size_t)2 * WAVES * MQ * 16 * 4;
-    auto kern = mqa_kernel<WAVES, MQ>;
+    auto kern = mqa_kernel<WAVES, MQ, NTK>;
     if (smem > 65536) {
         static bool done = false;
         if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
@@ -256,12 +290,12 @@ int launch_mqa_inst(const AttnP& p, hipStream_t s) {
 }  // namespace
 
 int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s) {
-    if (p.rows <= 0 || p.keys <= 0 || p.ldvt < ((p.keys + 63) / 64) * 64) return 1;
-    if (waves == 8) return launch_mqa_inst<8, 1>(p, s);
-    if (waves == 4) return launch_mqa_inst<4, 2>(p, s);
+    if (p.rows <= 0 || p.keys <= 0 || (p.ldvt & 63) || p.ldvt < ((p.keys + 63) / 64) * 64) return 1;
+    if (waves == 8) return launch_mqa_inst<4, 1, 4>(p, s);      // suffix pass: few rows, one row tile per workgroup
+    if (waves == 4) return launch_mqa_inst<4, 2, 2>(p, s);
     return 2;
 }
 
-void launch_vision_attention(const bf16_t* qk, const bf16_t* vt, bf16_t* out, int views, hipStream_t s) {
-    hipLaunchKernelGGL(vision_attn_kernel, dim3(views * 16 * 4), dim3(256), 0, s, qk, vt, out);
+void launch_vision_attention(const bf16_t* q, const bf16_t* k, const bf16_t* vt, bf16_t* out, int views, hipStream_t s) {
+    hipLaunchKernelGGL(vision_attn_kernel, dim3(views * 16 * 4), dim3(256), 0, s, q, k, vt, out);
 }

@@ -48,6 +48,20 @@ RTVLA_DEVICE int xcd_remap(int bid, int total) {
     return xcd * q + (xcd < r ? xcd : r) + idx;
 }
 
+// Fragment-tiled activation layout: a [rows][cols] matrix (cols a multiple of 32) stored as MFMA
+// operand fragments, tile (row/16, col/32) = 64 lanes x 8 bf16 with lane = row%16 + 16*((col%32)/8).
+// A wave reads one fragment as one contiguous 1 KB load (lane l takes bytes 16 l .. 16 l + 15).
+RTVLA_DEVICE size_t ft_index(int row, int col, int cols32) {
+    return ((size_t)((row >> 4) * cols32 + (col >> 5)) * 64 + (row & 15) + 16 * ((col & 31) >> 3)) * 8 + (col & 7);
+}
+// Transposed-V layout for attention: element (d, key) of V^T, tile (d/16, key/32); inside a tile the
+// 32 keys are permuted so that lane 16 g + r, register j holds key 4 g + (j & 3) + 16 (j >> 2): the
+// order in which the probabilities come out of the S^T = K Q^T accumulators.
+RTVLA_DEVICE size_t vt_index(int d, int key, int keys32) {
+    const int mm = key & 31;
+    return ((size_t)((d >> 4) * keys32 + (key >> 5)) * 64 + (d & 15) + 16 * ((mm & 15) >> 2)) * 8 + 4 * (mm >> 4) + (mm & 3);
+}
+
 RTVLA_DEVICE float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);

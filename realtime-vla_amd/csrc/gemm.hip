@@ -15,7 +15,7 @@ namespace {
 template <int EPI> struct EpiTraits { static constexpr bool dual = (EPI == EPI_GEGLU); };
 
 template <int WN, int MT, int NT, int EPI>
-__global__ __launch_bounds__(WN * 64)
+__global__ __launch_bounds__(WN * 64) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int stages_per_split) {
     constexpr int NTH = WN * 64;
     constexpr int BM = MT * 16;
@@ -50,8 +50,6 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         const int tc = min(t, p.N16 - 1);
         bptr[j] = base + (size_t)tc * p.K32p * 512 + lane * 8;
     }
-    // m-tiles of this block that hold valid rows
-    const int mt_valid = min(MT, (p.M - m0 + 15) >> 4);
 
     f32x4 acc[MT][NT];
 #pragma unroll
@@ -62,66 +60,79 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
     uint4 areg[AIT];
     bf16x8 breg0[NT][2], breg1[NT][2];
 
-    auto load_a = [&](int s) {
+    auto load_a = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < AIT; ++it) {
-            const int c = it * NTH + tid;
-            if (A_CHUNKS % NTH == 0 || c < A_CHUNKS) {
-                const int row = c >> 3, kc = c & 7;
-                const int gr = min(m0 + row, p.a_rows - 1);
-                areg[it] = *(const uint4*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
-            }
+            // a ragged last round re-reads the final chunk instead of branching
+            const int c = min(it * NTH + tid, A_CHUNKS - 1);
+            const int row = c >> 3, kc = c & 7;
+            const int gr = min(m0 + row, p.a_rows - 1);
+            areg[it] = *(const uint4*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
         }
     };
-    auto store_a = [&](int buf) {
+    auto store_a = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < AIT; ++it) {
-            const int c = it * NTH + tid;
-            if (A_CHUNKS % NTH == 0 || c < A_CHUNKS) {
-                const int row = c >> 3, kc = c & 7;
-                const int off = ((((row >> 4) * 2 + (kc >> 2)) * 64) + (row & 15) + 16 * (kc & 3)) * 8;
-                *(uint4*)(lds + buf * STAGE_ELEMS + off) = areg[it];
-            }
+            const int c = min(it * NTH + tid, A_CHUNKS - 1);      // duplicates write identical data
+            const int row = c >> 3, kc = c & 7;
+            const int off = ((((row >> 4) * 2 + (kc >> 2)) * 64) + (row & 15) + 16 * (kc & 3)) * 8;
+            *(uint4*)(lds + buf * STAGE_ELEMS + off) = areg[it];
         }
     };
-    auto load_b = [&](int s, bf16x8 (&br)[NT][2]) {
+    auto load_b = [&](int s, bf16x8 (&br)[NT][2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < NT; ++j)
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
                 br[j][kk] = *(const bf16x8*)(bptr[j] + (size_t)(s * 2 + kk) * 512);
     };
-    auto compute = [&](int buf, bf16x8 (&br)[NT][2]) {
+    auto compute = [&](int buf, bf16x8 (&br)[NT][2]) __attribute__((always_inline)) {
         const bf16_t* base = lds + buf * STAGE_ELEMS + lane * 8;
+        // all A fragments of the stage are requested from LDS before the first MFMA waits on one
+        bf16x8 af[2][MT];
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                if (i < mt_valid) {
-                    const bf16x8 a = *(const bf16x8*)(base + (i * 2 + kk) * 512);
+            for (int i = 0; i < MT; ++i) af[kk][i] = *(const bf16x8*)(base + (i * 2 + kk) * 512);
 #pragma unroll
-                    for (int j = 0; j < NT; ++j) acc[i][j] = mfma16(br[j][kk], a, acc[i][j]);
-                }
-            }
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[i][j] = mfma16(br[j][kk], af[kk][i], acc[i][j]);
+        // instruction order for the scheduler: PRE fragment reads ahead, then NT MFMAs per further read
+        constexpr int PRE = 4;
+        __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
+#pragma unroll
+        for (int t = 0; t < 2 * MT - PRE; ++t) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+#pragma unroll
+        for (int t = 0; t < PRE; ++t) __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
     };
 
+    // stages come in pairs (the host guarantees an even count per split) so that the two register
+    // sets alternate without a runtime index; the loop body is branch free: the last round's
+    // prefetch re-reads a valid stage instead of being skipped
     if (s_begin < s_end) {
         load_a(s_begin);
         load_b(s_begin, breg0);
         store_a(0);
         __syncthreads();
         for (int s = s_begin; s < s_end; s += 2) {
-            const bool more1 = s + 1 < s_end;
-            if (more1) { load_a(s + 1); load_b(s + 1, breg1); }
+            load_a(s + 1); load_b(s + 1, breg1);
+            __builtin_amdgcn_sched_barrier(0);           // next stage's loads fly under this stage's MFMAs
             compute(0, breg0);
-            if (more1) store_a(1);
+            __builtin_amdgcn_sched_barrier(0);
+            store_a(1);
             __syncthreads();
-            if (!more1) break;
-            const bool more2 = s + 2 < s_end;
-            if (more2) { load_a(s + 2); load_b(s + 2, breg0); }
+            const int s2 = min(s + 2, s_end - 2);
+            load_a(s2); load_b(s2, breg0);
+            __builtin_amdgcn_sched_barrier(0);
             compute(1, breg1);
-            if (more2) store_a(0);
+            __builtin_amdgcn_sched_barrier(0);
+            store_a(0);
             __syncthreads();
         }
     }
@@ -130,7 +141,7 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int m = m0 + i * 16 + r;
-        if (i >= mt_valid || m >= p.M) continue;
+        if (m >= p.M) continue;
 #pragma unroll
         for (int j = 0; j < HALF; ++j) {
             const int t = tile_of[j];
@@ -167,25 +178,27 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
                     const f32x4 w = v;
                     v[0] = w[0] * c0 - w[1] * s0; v[1] = w[1] * c0 + w[0] * s0;
                     v[2] = w[2] * c1 - w[3] * s1; v[3] = w[3] * c1 + w[2] * s1;
-                    if (n0 < 2048) store4(p.q + (size_t)m * 2048 + n0, pack4(v));
-                    else store4(p.k + (size_t)m * 256 + (n0 - 2048), pack4(v));
+                    // Q rows are token*8 + head; Q and K are kept fragment-tiled for the attention kernel
+                    if (n0 < 2048) store4(p.q + ft_index(m * 8 + (n0 >> 8), n0 & 255, 8), pack4(v));
+                    else store4(p.k + ft_index(m, n0 - 2048, 8), pack4(v));
                 } else {
                     const int d = n0 - 2304;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) p.vt[(size_t)(d + e) * p.ldvt + m] = f2bf(v[e]);
+                    for (int e = 0; e < 4; ++e) p.vt[vt_index(d + e, m, p.ldvt >> 5)] = f2bf(v[e]);
                 }
             } else if constexpr (EPI == EPI_VIS_QKV) {
                 const bf16x4 b = load4(p.bias + n0);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] += bf2f(b[e]);
-                if (n0 < 2304) {
-                    store4(p.out + (size_t)m * p.ldo + n0, pack4(v));
-                } else {
-                    const int c = n0 - 2304, head = c / 72, d = c - head * 72;
-                    const int view = m >> 8, tok = m & 255;
-                    bf16_t* dst = p.vt + ((size_t)(view * 16 + head) * 80 + d) * 256 + tok;
+                // per (view, head): Q and K as fragment-tiled [256 tokens][96] (72 padded), V^T as [80][256]
+                const int which = n0 / 1152, c = n0 - which * 1152, head = c / 72, d = c - head * 72;
+                const int view = m >> 8, tok = m & 255;
+                const size_t vh = (size_t)(view * 16 + head);
+                if (which == 0) store4(p.q + vh * (256 * 96) + ft_index(tok, d, 3), pack4(v));
+                else if (which == 1) store4(p.k + vh * (256 * 96) + ft_index(tok, d, 3), pack4(v));
+                else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) dst[(size_t)e * 256] = f2bf(v[e]);
+                    for (int e = 0; e < 4; ++e) p.vt[vh * (80 * 256) + vt_index(d + e, tok, 8)] = f2bf(v[e]);
                 }
             }
         }
@@ -202,6 +215,7 @@ int launch_cfg(const GemmP& p, hipStream_t s) {
     const int nsplit = p.nsplit < 1 ? 1 : p.nsplit;
     const int sps = (stages_total + nsplit - 1) / nsplit;
     if ((nsplit - 1) * sps >= stages_total) return 3;      // an empty split would leave its partial unwritten
+    if ((sps & 1) || (stages_total & 1)) return 3;          // the kernel consumes K stages in pairs
     GemmP q = p; q.nsplit = nsplit;
     const size_t smem = (size_t)2 * BM * 64 * sizeof(bf16_t);
     auto kern = gemm_mfma_kernel<WN, MT, NT, EPI>;

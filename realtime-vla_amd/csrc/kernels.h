@@ -12,8 +12,8 @@
 // tile (nb, kb) holds the 16 columns nb*16.. and 32 rows kb*32.. as 64 lanes x 8 bf16,
 // lane l = 16 g + r carrying W[kb*32 + 8 g + j][nb*16 + r], j = 0..7.  Tiles are stored
 // [nb][kb] so that one column block streams contiguously along K.  K is padded to a
-// multiple of 64 and N to a multiple of 16 with zeros.
-static inline int k32_padded(int K) { return ((K + 63) / 64) * 2; }
+// multiple of 128 (the GEMM consumes 64-wide K stages in pairs) and N to a multiple of 16 with zeros.
+static inline int k32_padded(int K) { return ((K + 127) / 128) * 4; }
 static inline int n16_tiles(int N) { return (N + 15) / 16; }
 static inline size_t tiled_elems(int K, int N) { return (size_t)n16_tiles(N) * k32_padded(K) * 512; }
 
@@ -71,6 +71,8 @@ enum SkinnyEpilogue {
 enum SkinnyNorm { SN_NONE = 0, SN_RMS, SN_ADARMS };
 struct SkinnyP {
     const bf16_t* A; int lda; int M;           // valid rows (<= 64)
+    int a_tiled; int a_row0;                   // A in the fragment-tiled layout; first row inside it
+    int out_tiled; int out_row0;               // same for `out`
     const bf16_t* B0; const bf16_t* B1; int K; int N16; int K32p;
     int norm; const bf16_t* style;             // SN_ADARMS: [scale | shift | gate] each K wide
     float eps;
@@ -82,15 +84,17 @@ struct SkinnyP {
 int launch_skinny(const SkinnyP& p, int epi, hipStream_t s);
 
 // out[m][n] = act(bias[n] + sum_k x[m][k] W[k][n]) for tiny K (<= 64), W in its original layout
+// (`out` fragment-tiled with first row out_row0 when out_tiled)
 void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t* bias, bf16_t* out, int ldo,
-                         int M, int K, int N, int act_silu, hipStream_t s);
+                         int M, int K, int N, int act_silu, int out_tiled, int out_row0, hipStream_t s);
 
 // ----- attention --------------------------------------------------------------------------
 struct AttnP {
-    const bf16_t* q; int ldq;        // [rows][ldq]
-    const bf16_t* k; int ldk;        // [keys][ldk]
-    const bf16_t* vt; int ldvt;      // [d][ldvt] (keys contiguous)
-    bf16_t* out; int ldo;            // [rows][ldo]
+    const bf16_t* q;                 // fragment-tiled [rows padded to the workgroup tile][256]
+    const bf16_t* k;                 // fragment-tiled [keys padded to 64][256]
+    const bf16_t* vt; int ldvt;      // permuted-key tiled V^T [256][ldvt], ldvt = keys padded to 64
+    bf16_t* out; int ldo;            // row-major or fragment-tiled [rows][256] (out_tiled)
+    int out_tiled;
     int rows, keys;
     float scale;
     // masking: key j is visible to row r iff
@@ -99,8 +103,8 @@ struct AttnP {
     int prefix_alloc; const int* valid_len; int state_rows;
 };
 int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s);
-// SigLIP attention: qk [views*256][2304] (Q | K, 16 heads x 72), vt [views*16][80][256]
-void launch_vision_attention(const bf16_t* qk, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);
+// SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major
+void launch_vision_attention(const bf16_t* q, const bf16_t* k, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);
 
 // ----- small helpers ------------------------------------------------------------------------
 void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hipStream_t s);

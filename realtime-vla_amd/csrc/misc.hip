@@ -116,14 +116,15 @@ __global__ void im2col_kernel(const bf16_t* __restrict__ img, bf16_t* __restrict
 // tiny-K linear: one thread per output element, W[K][N] row-major (coalesced over n)
 __global__ void small_linear_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ W,
                                     const bf16_t* __restrict__ bias, bf16_t* __restrict__ out, int ldo,
-                                    int M, int K, int N, int act_silu) {
+                                    int M, int K, int N, int act_silu, int out_tiled, int out_row0) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= M * N) return;
     const int m = idx / N, n = idx - m * N;
     float acc = bias ? bf2f(bias[n]) : 0.f;
     for (int k = 0; k < K; ++k) acc += bf2f(x[(size_t)m * ldx + k]) * bf2f(W[(size_t)k * N + n]);
     if (act_silu) acc = siluf(acc);
-    out[(size_t)m * ldo + n] = f2bf(acc);
+    if (out_tiled) out[ft_index(m + out_row0, n, ldo >> 5)] = f2bf(acc);
+    else out[(size_t)m * ldo + n] = f2bf(acc);
 }
 
 // RoPE table rows [cos_i, sin_i] interleaved for positions pos0 .. pos0 + count - 1, where
@@ -189,9 +190,9 @@ void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hi
 }
 
 void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t* bias, bf16_t* out, int ldo,
-                         int M, int K, int N, int act_silu, hipStream_t s) {
+                         int M, int K, int N, int act_silu, int out_tiled, int out_row0, hipStream_t s) {
     const int total = M * N;
-    hipLaunchKernelGGL(small_linear_kernel, dim3((total + 255) / 256), dim3(256), 0, s, x, ldx, W, bias, out, ldo, M, K, N, act_silu);
+    hipLaunchKernelGGL(small_linear_kernel, dim3((total + 255) / 256), dim3(256), 0, s, x, ldx, W, bias, out, ldo, M, K, N, act_silu, out_tiled, out_row0);
 }
 
 void launch_rope_table(bf16_t* table, const int* dyn_start, int start, int count, hipStream_t s) {

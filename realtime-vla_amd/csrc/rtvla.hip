@@ -81,6 +81,14 @@ struct rtvla_ctx {
     }
     bf16_t* TW(const char* n, int layer = 0) { const WsBuf& b = BI(n); return (bf16_t*)(ws + b.offset) + (size_t)b.ld * layer; }
 
+    int only = -1;                 // >= 0: enqueue only the launch with this index (per-kernel timing)
+    std::string last_name;
+    bool want(const char* what) {
+        const bool yes = only < 0 || only == launches;
+        if (yes) last_name = what;
+        if (!yes) ++launches;
+        return yes;
+    }
     void note(int rc, const char* what) {
         ++launches;
         if (rc != 0 && status == 0) { status = RTVLA_ERR_DEVICE; err = std::string("launch failed: ") + what + " (code " + std::to_string(rc) + ")"; }
@@ -112,7 +120,7 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
         for (int sp : splits) {
             if (sp > 1 && !splittable) break;
             const int sps = (stages + sp - 1) / sp;
-            if ((sp - 1) * sps >= stages) continue;
+            if ((sp - 1) * sps >= stages || (sps & 1)) continue;
             const int blocks = mb * nb * sp;
             const int rounds = (blocks + 255) / 256;
             double t = rounds * (mt * (sps + 1.0) * 4.0 * 2 * 16 / 2400.0 + 1.5);       // us: MFMA cycles at 2.4 GHz + fixed
@@ -228,25 +236,25 @@ int build_tables(rtvla_ctx* c) {
     c->add_buf("vision_patches", S_v, PATCH_LD, PATCH_LD);
     c->add_buf("vision_x", S_v, 1152, 1152);
     c->add_buf("vision_x_norm", S_v, 1152, 1152);
-    c->add_buf("vision_QK", S_v, 2304, 2304);
-    c->add_buf("vision_Vt", v * 16 * 80, 256, 256);
+    c->add_buf("vision_Q", v * 16, 256 * 96, 256 * 96);          // fragment-tiled [256][96] per (view, head)
+    c->add_buf("vision_K", v * 16, 256 * 96, 256 * 96);
+    c->add_buf("vision_Vt", v * 16, 80 * 256, 80 * 256);         // tiled V^T [80][256] per (view, head)
     c->add_buf("vision_attn", S_v, 1152, 1152);
     c->add_buf("vision_hidden", S_v, 4304, VHID_LD);
     c->add_buf("encoder_x", S_e, 2048, 2048);
     c->add_buf("encoder_x_norm", S_e, 2048, 2048);
-    c->add_buf("encoder_Q", S_e, 2048, 2048);
+    c->add_buf("encoder_Q", ((8 * S_e + 31) / 32) * 32, 256, 256);   // fragment-tiled, rows = token*8 + head
     c->add_buf("encoder_attn", S_e, 2048, 2048);
     c->add_buf("encoder_hidden", S_e, 16384, 16384);
-    c->add_buf("encoder_K", L * c->keys, 256, 256);
-    c->add_buf("encoder_Vt", L * 256, c->keys, c->keys_pad);
-    c->add_buf("decoder_x", S_d, 1024, 1024);
-    c->add_buf("decoder_x_buf", std::max<int64_t>(ch, 16), 1024, 1024);
-    c->add_buf("decoder_state_buf", 1, 1024, 1024);
-    c->add_buf("decoder_q_buf", S_d, 2048, 2048);
-    c->add_buf("decoder_attn", S_d, 2048, 2048);
-    c->add_buf("decoder_hidden", S_d, 4096, 4096);
+    c->add_buf("encoder_K", L * c->keys_pad, 256, 256);           // fragment-tiled [keys_pad][256] per layer
+    c->add_buf("encoder_Vt", L * 256, c->keys_pad, c->keys_pad);  // tiled V^T [256][keys_pad] per layer
+    c->add_buf("decoder_x", 64, 1024, 1024);                      // the decoder_* activations are fragment-tiled
+    c->add_buf("decoder_x_buf", 64, 1024, 1024);
+    c->add_buf("decoder_q_buf", 512, 256, 256);
+    c->add_buf("decoder_attn", 64, 2048, 2048);
+    c->add_buf("decoder_hidden", 64, 4096, 4096);
     if (pi05) {
-        c->add_buf("decoder_time_emb", d.num_steps, 1024, 1024);
+        c->add_buf("decoder_time_emb", 64, 1024, 1024);           // fragment-tiled, one row per step
         c->add_buf("decoder_style_attn", d.num_steps, L * 3072, L * 3072);
         c->add_buf("decoder_style_ffn", d.num_steps, L * 3072, L * 3072);
         c->add_buf("decoder_style_final", d.num_steps, 3072, 3072);
@@ -276,7 +284,7 @@ struct Sched {
             p.partial = c->B<float>("splitk_partial"); p.ldp = N; p.pstride = (size_t)M * N;
         }
         last_split = tc.nsplit;
-        c->note(launch_gemm(p, epi, tc.tile, s), what);
+        if (c->want(what)) c->note(launch_gemm(p, epi, tc.tile, s), what);
     }
     int last_split = 1;
 
@@ -286,12 +294,12 @@ struct Sched {
         p.partial = c->B<float>("splitk_partial"); p.pstride = (size_t)M * N; p.ldp = N; p.nsplit = nsplit;
         p.bias = bias; p.res = res; p.ldr = ldr; p.x = x; p.ldx = ldx; p.xn = xn; p.ldxn = ldxn;
         p.M = M; p.N = N; p.norm = norm; p.nw = nw; p.nb = nb; p.eps = eps;
-        c->note(launch_reduce(p, s), what);
+        if (c->want(what)) c->note(launch_reduce(p, s), what);
     }
 
     void vision_embed() {
         const int S_v = c->S_v;
-        launch_im2col(c->W("observation_images_normalized"), c->B("vision_patches"), PATCH_LD, d.num_views, s); c->note(0, "im2col");
+        if (c->want("im2col")) { launch_im2col(c->W("observation_images_normalized"), c->B("vision_patches"), PATCH_LD, d.num_views, s); c->note(0, "im2col"); }
         GemmP e{}; e.out = c->B("vision_x"); e.ldo = 1152; e.bias = c->W("vision_patch_embedding_b");
         e.res = c->W("vision_position_embedding"); e.ldr = 1152; e.res_mod = 256;
         gemm(c->B("vision_patches"), PATCH_LD, S_v, S_v, c->TW("t_vision_patch_embedding_w"), nullptr, 588, 1152, EPI_PATCH, e, "patch embed");
@@ -301,9 +309,9 @@ struct Sched {
 
     void vision_layer(int i) {
         const int S_v = c->S_v, V = d.vision_layers;
-        GemmP e{}; e.out = c->B("vision_QK"); e.ldo = 2304; e.bias = c->W("vision_attn_qkv_b", 3456, i); e.vt = c->B("vision_Vt");
+        GemmP e{}; e.bias = c->W("vision_attn_qkv_b", 3456, i); e.q = c->B("vision_Q"); e.k = c->B("vision_K"); e.vt = c->B("vision_Vt");
         gemm(c->B("vision_x_norm"), 1152, S_v, S_v, c->TW("t_vision_attn_qkv_w", i), nullptr, 1152, 3456, EPI_VIS_QKV, e, "vision qkv");
-        launch_vision_attention(c->B("vision_QK"), c->B("vision_Vt"), c->B("vision_attn"), d.num_views, s); c->note(0, "vision attn");
+        if (c->want("vision attn")) { launch_vision_attention(c->B("vision_Q"), c->B("vision_K"), c->B("vision_Vt"), c->B("vision_attn"), d.num_views, s); c->note(0, "vision attn"); }
         gemm(c->B("vision_attn"), 1152, S_v, S_v, c->TW("t_vision_attn_o_w", i), nullptr, 1152, 1152, EPI_PARTIAL, GemmP{}, "vision o");
         reduce(S_v, 1152, c->W("vision_attn_o_b", 1152, i), c->B("vision_x"), 1152, c->B("vision_x"), 1152, c->B("vision_x_norm"), 1152,
                NORM_LAYER, c->W("vision_pre_ffn_norm_w", 1152, i), c->W("vision_pre_ffn_norm_b", 1152, i), 1e-5f, last_split, "vision o reduce");
@@ -322,13 +330,12 @@ struct Sched {
         GemmP e{}; e.out = c->B("encoder_x"); e.ldo = 2048; e.bias = c->W("encoder_multi_modal_projector_b");
         gemm(c->B("vision_x_norm"), 1152, S_v, S_v, c->TW("t_encoder_multi_modal_projector_w"), nullptr, 1152, 2048, EPI_BIAS, e, "projector");
         if (!pi05 && d.prompt_len > 0) {
-            launch_copy_rows(c->W("language_embeds"), 2048, c->B("encoder_x") + (size_t)S_v * 2048, 2048, d.prompt_len, 2048, s);
-            c->note(0, "prompt rows");
+            if (c->want("prompt rows")) { launch_copy_rows(c->W("language_embeds"), 2048, c->B("encoder_x") + (size_t)S_v * 2048, 2048, d.prompt_len, 2048, s); c->note(0, "prompt rows"); }
         }
         reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, nullptr, 0, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, 0, "prefix rms0");
     }
 
-    bf16_t* Kc(int i) { return c->B("encoder_K") + (size_t)i * c->keys * 256; }
+    bf16_t* Kc(int i) { return c->B("encoder_K") + (size_t)i * c->keys_pad * 256; }
     bf16_t* Vt(int i) { return c->B("encoder_Vt") + (size_t)i * 256 * c->keys_pad; }
     const int* valid_len() { return pi05 ? (const int*)c->tensors[c->tindex.at("valid_encoder_len")].ptr : nullptr; }
 
@@ -338,10 +345,10 @@ struct Sched {
         gemm(c->B("encoder_x_norm"), 2048, S_e, S_e, c->TW("t_encoder_attn_qkv_w", i), nullptr, 2048, 2560, EPI_QKV_ROPE, e, "prefix qkv");
         if (i == L - 1) return;                      // the last layer only fills the KV cache
         AttnP a{};
-        a.q = c->B("encoder_Q"); a.ldq = 256; a.k = Kc(i); a.ldk = 256; a.vt = Vt(i); a.ldvt = c->keys_pad;
-        a.out = c->B("encoder_attn"); a.ldo = 256; a.rows = 8 * S_e; a.keys = S_e; a.scale = 0.0625f;
+        a.q = c->B("encoder_Q"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
+        a.out = c->B("encoder_attn"); a.ldo = 256; a.out_tiled = 0; a.rows = 8 * S_e; a.keys = S_e; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = 0;
-        c->note(launch_mqa_attention(a, 4, s), "prefix attn");
+        if (c->want("prefix attn")) c->note(launch_mqa_attention(a, 4, s), "prefix attn");
         gemm(c->B("encoder_attn"), 2048, S_e, S_e, c->TW("t_encoder_attn_o_w", i), nullptr, 2048, 2048, EPI_PARTIAL, GemmP{}, "prefix o");
         reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix o reduce");
         GemmP g{}; g.out = c->B("encoder_hidden"); g.ldo = 16384;
@@ -350,34 +357,42 @@ struct Sched {
         reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix down reduce");
     }
 
+    // action-expert activations live in the fragment-tiled layout (64 rows x cols)
     void skinny(const bf16_t* A, int lda, int M, const bf16_t* B0, const bf16_t* B1, int K, int N, int norm, const bf16_t* style,
                 int epi, SkinnyP extra, const char* what) {
         SkinnyP p = extra;
         p.A = A; p.lda = lda; p.M = M; p.B0 = B0; p.B1 = B1; p.K = K; p.N16 = n16_tiles(N); p.K32p = k32_padded(K);
         p.norm = norm; p.style = style; p.eps = 1e-6f;
-        c->note(launch_skinny(p, epi, s), what);
+        if (c->want(what)) c->note(launch_skinny(p, epi, s), what);
+    }
+    static SkinnyP tiled_io(int a_row0 = 0, int out_row0 = 0) {
+        SkinnyP p{}; p.a_tiled = 1; p.a_row0 = a_row0; p.out_tiled = 1; p.out_row0 = out_row0; return p;
     }
 
-    void suffix_init() {
-        if (pi05) return;
-        launch_small_linear(c->W("observation_state_normalized"), 32, c->W("decoder_state_in_proj_w"), c->W("decoder_state_in_proj_b"),
-                            c->B("decoder_state_buf"), 1024, 1, 32, 1024, 0, s);
-        c->note(0, "state proj");
-    }
+    void suffix_init() {}
 
     void suffix_step_begin(int t) {
         const int ch = d.chunk_size;
         if (!pi05) {
-            launch_copy_rows(c->B("decoder_state_buf"), 1024, c->B("decoder_x"), 1024, 1, 1024, s); c->note(0, "state row");
-            launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_fused_in_proj_w"),
-                                c->W("decoder_action_fused_time_biases", 1024, t % 10), c->B("decoder_x_buf"), 1024, ch, 32, 1024, 1, s);
-            c->note(0, "action in");
-            SkinnyP e{}; e.out = c->B("decoder_x") + 1024; e.ldo = 1024; e.bias = c->W("decoder_action_mlp_b");
+            // state token -> row 0 (re-projected every step: the residual stream is updated in place)
+            if (c->want("state proj")) {
+                launch_small_linear(c->W("observation_state_normalized"), 32, c->W("decoder_state_in_proj_w"), c->W("decoder_state_in_proj_b"),
+                                    c->B("decoder_x"), 1024, 1, 32, 1024, 0, 1, 0, s);
+                c->note(0, "state proj");
+            }
+            if (c->want("action in")) {
+                launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_fused_in_proj_w"),
+                                    c->W("decoder_action_fused_time_biases", 1024, t % 10), c->B("decoder_x_buf"), 1024, ch, 32, 1024, 1, 1, 0, s);
+                c->note(0, "action in");
+            }
+            SkinnyP e = tiled_io(0, 1); e.out = c->B("decoder_x"); e.ldo = 1024; e.bias = c->W("decoder_action_mlp_b");
             skinny(c->B("decoder_x_buf"), 1024, ch, c->TW("t_decoder_action_mlp_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS, e, "action mlp");
         } else {
-            launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_in_proj_w"), c->W("decoder_action_in_proj_b"),
-                                c->B("decoder_x"), 1024, ch, 32, 1024, 0, s);
-            c->note(0, "action in");
+            if (c->want("action in")) {
+                launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_in_proj_w"), c->W("decoder_action_in_proj_b"),
+                                    c->B("decoder_x"), 1024, ch, 32, 1024, 0, 1, 0, s);
+                c->note(0, "action in");
+            }
         }
     }
 
@@ -386,27 +401,28 @@ struct Sched {
         const int norm = pi05 ? SN_ADARMS : SN_RMS;
         const bf16_t* st_attn = pi05 ? c->B("decoder_style_attn") + ((size_t)t * L + i) * 3072 : nullptr;
         const bf16_t* st_ffn = pi05 ? c->B("decoder_style_ffn") + ((size_t)t * L + i) * 3072 : nullptr;
-        SkinnyP q{}; q.rope = c->W("decoder_rope_weights"); q.q = c->B("decoder_q_buf"); q.k = Kc(i); q.vt = Vt(i); q.ldvt = c->keys_pad; q.kv_row0 = S_e;
+        SkinnyP q = tiled_io(); q.rope = c->W("decoder_rope_weights"); q.q = c->B("decoder_q_buf"); q.k = Kc(i); q.vt = Vt(i); q.ldvt = c->keys_pad; q.kv_row0 = S_e;
         skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_attn_qkv_w", i), nullptr, 1024, 2560, norm, st_attn, SK_QKV_ROPE, q, "suffix qkv");
         AttnP a{};
-        a.q = c->B("decoder_q_buf"); a.ldq = 256; a.k = Kc(i); a.ldk = 256; a.vt = Vt(i); a.ldvt = c->keys_pad;
-        a.out = c->B("decoder_attn"); a.ldo = 256; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
+        a.q = c->B("decoder_q_buf"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
+        a.out = c->B("decoder_attn"); a.ldo = 256; a.out_tiled = 1; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
-        c->note(launch_mqa_attention(a, 8, s), "suffix attn");
-        SkinnyP o{}; o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
+        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, 8, s), "suffix attn");
+        SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
         skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
-        SkinnyP g{}; g.out = c->B("decoder_hidden"); g.ldo = 4096;
+        SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 4096;
         skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_ffn_gate_w", i), c->TW("t_decoder_ffn_up_w", i), 1024, 4096, norm, st_ffn, SK_GEGLU, g, "suffix geglu");
-        SkinnyP dn{}; dn.out = c->B("decoder_x"); dn.ldo = 1024; dn.gate = pi05 ? st_ffn + 2048 : nullptr;
+        SkinnyP dn = tiled_io(); dn.out = c->B("decoder_x"); dn.ldo = 1024; dn.gate = pi05 ? st_ffn + 2048 : nullptr;
         skinny(c->B("decoder_hidden"), 4096, S_d, c->TW("t_decoder_ffn_down_w", i), nullptr, 4096, 1024, SN_NONE, nullptr, SK_RES, dn, "suffix down");
     }
 
     void suffix_step_end(int t) {
         const int ch = d.chunk_size;
-        SkinnyP e{}; e.out = c->W("diffusion_noise"); e.ldo = 32;
+        SkinnyP e{}; e.a_tiled = 1; e.out = c->W("diffusion_noise"); e.ldo = 32;       // noise stays row-major [chunk][32]
         if (!pi05) {
+            e.a_row0 = 1;                                                               // action rows follow the state token
             e.bias = c->W("decoder_action_fused_out_proj_b");
-            skinny(c->B("decoder_x") + 1024, 1024, ch, c->TW("t_decoder_out_proj_w"), nullptr, 1024, 32, SN_RMS, nullptr, SK_RES, e, "euler");
+            skinny(c->B("decoder_x"), 1024, ch, c->TW("t_decoder_out_proj_w"), nullptr, 1024, 32, SN_RMS, nullptr, SK_RES, e, "euler");
         } else {
             e.bias = c->B("decoder_out_proj_b_scaled");
             skinny(c->B("decoder_x"), 1024, ch, c->TW("t_decoder_out_proj_w"), nullptr, 1024, 32, SN_ADARMS,
@@ -485,18 +501,18 @@ struct Sched {
         tile("decoder_pre_ffn_norm_mod_w", "t_decoder_pre_ffn_norm_mod_w", 1024, 3072, L);
         tile("decoder_final_norm_mod_w", "t_decoder_final_norm_mod_w", 1024, 3072, 1);
         const int T = d.num_steps;
-        SkinnyP e{}; e.out = c->B("decoder_x_buf"); e.ldo = 1024; e.bias = c->W("decoder_time_mlp_in_b");
+        SkinnyP e{}; e.out_tiled = 1; e.out = c->B("decoder_x_buf"); e.ldo = 1024; e.bias = c->W("decoder_time_mlp_in_b");
         skinny(c->W("decoder_time_embeds"), 1024, T, c->TW("t_decoder_time_mlp_in_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS_SILU, e, "time mlp in");
-        e.out = c->B("decoder_time_emb"); e.bias = c->W("decoder_time_mlp_out_b");
+        e.a_tiled = 1; e.out = c->B("decoder_time_emb"); e.bias = c->W("decoder_time_mlp_out_b");
         skinny(c->B("decoder_x_buf"), 1024, T, c->TW("t_decoder_time_mlp_out_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS_SILU, e, "time mlp out");
         for (int i = 0; i < L; ++i) {
-            SkinnyP m{}; m.ldo = L * 3072;
+            SkinnyP m{}; m.a_tiled = 1; m.ldo = L * 3072;
             m.out = c->B("decoder_style_attn") + (size_t)i * 3072; m.bias = c->W("decoder_pre_attn_norm_mod_b", 3072, i);
             skinny(c->B("decoder_time_emb"), 1024, T, c->TW("t_decoder_pre_attn_norm_mod_w", i), nullptr, 1024, 3072, SN_NONE, nullptr, SK_BIAS, m, "style attn");
             m.out = c->B("decoder_style_ffn") + (size_t)i * 3072; m.bias = c->W("decoder_pre_ffn_norm_mod_b", 3072, i);
             skinny(c->B("decoder_time_emb"), 1024, T, c->TW("t_decoder_pre_ffn_norm_mod_w", i), nullptr, 1024, 3072, SN_NONE, nullptr, SK_BIAS, m, "style ffn");
         }
-        SkinnyP f{}; f.ldo = 3072; f.out = c->B("decoder_style_final"); f.bias = c->W("decoder_final_norm_mod_b");
+        SkinnyP f{}; f.a_tiled = 1; f.ldo = 3072; f.out = c->B("decoder_style_final"); f.bias = c->W("decoder_final_norm_mod_b");
         skinny(c->B("decoder_time_emb"), 1024, T, c->TW("t_decoder_final_norm_mod_w"), nullptr, 1024, 3072, SN_NONE, nullptr, SK_BIAS, f, "style final");
     }
 };
@@ -682,6 +698,33 @@ int rtvla_time_stage(rtvla_ctx* c, int stage, int layer, int step, int iters, vo
         else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / iters; }
     }
     hipEventDestroy(a); hipEventDestroy(b);
+    if (rc) return rc;
+    return c->status;
+}
+
+int rtvla_time_launch(rtvla_ctx* c, int stage, int layer, int step, int launch_index, int iters, void* stream,
+                      float* mean_ms, char* name_out, size_t name_cap) {
+    if (int rc = check_ready(c, true)) return rc;
+    if (iters < 1 || !mean_ms || launch_index < 0) return RTVLA_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    hipEvent_t a, b;
+    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
+    Sched sc(c, s);
+    c->status = 0; c->only = launch_index; c->last_name.clear();
+    c->launches = 0;
+    int rc = sc.stage(stage, layer, step);      // warm-up, also tells whether the index exists
+    if (!rc && c->launches <= launch_index) rc = c->fail(RTVLA_ERR_ARG, "launch index past the end of the stage");
+    if (!rc) {
+        hipEventRecord(a, s);
+        for (int i = 0; i < iters && !rc; ++i) { c->launches = 0; rc = sc.stage(stage, layer, step); }
+        hipEventRecord(b, s);
+        hipError_t e = hipEventSynchronize(b);
+        if (e != hipSuccess) rc = hip_fail(c, e, "time_launch");
+        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / iters; }
+    }
+    c->only = -1;
+    hipEventDestroy(a); hipEventDestroy(b);
+    if (name_out && name_cap) { strncpy(name_out, c->last_name.c_str(), name_cap - 1); name_out[name_cap - 1] = 0; }
     if (rc) return rc;
     return c->status;
 }

@@ -18,7 +18,7 @@ constexpr int SK_MTS = 4;      // 4 x 16 = 64 rows
 constexpr int SK_CH = 4;       // k32 blocks per A-prefetch chunk
 
 template <int NCH, int NORM, int EPI>
-__global__ __launch_bounds__(SK_WAVES * 64)
+__global__ __launch_bounds__(SK_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void skinny_kernel(SkinnyP p) {
     constexpr int KBW = NCH * SK_CH;
     constexpr bool DUAL = (EPI == SK_GEGLU);
@@ -45,11 +45,14 @@ void skinny_kernel(SkinnyP p) {
             for (int i = 0; i < KBW; ++i) b[1][i] = *(const bf16x8*)(bp1 + (size_t)i * 512);
         }
     }
+    // activation fragments: with the fragment-tiled layout (and no row offset) each is one
+    // contiguous 1 KB read; astep is the distance between consecutive k32 blocks of a row
     const bf16_t* arow[SK_MTS];
+    const int astep = p.a_tiled ? 512 : 32;
 #pragma unroll
     for (int mt = 0; mt < SK_MTS; ++mt) {
-        const int row = min(mt * 16 + r, p.M - 1);
-        arow[mt] = p.A + (size_t)row * p.lda + kb0 * 32 + 8 * g;
+        const int row = min(mt * 16 + r, p.M - 1) + p.a_row0;
+        arow[mt] = p.a_tiled ? p.A + ft_index(row, kb0 * 32 + 8 * g, p.lda >> 5) : p.A + (size_t)row * p.lda + kb0 * 32 + 8 * g;
     }
     f32x4 acc[NB][SK_MTS];
 #pragma unroll
@@ -62,13 +65,15 @@ void skinny_kernel(SkinnyP p) {
 #pragma unroll
         for (int mt = 0; mt < SK_MTS; ++mt)
 #pragma unroll
-            for (int i = 0; i < SK_CH; ++i) dst[mt][i] = *(const bf16x8*)(arow[mt] + (c * SK_CH + i) * 32);
+            for (int i = 0; i < SK_CH; ++i) dst[mt][i] = *(const bf16x8*)(arow[mt] + (c * SK_CH + i) * astep);
     };
     load_a(0, a[0]);
+    // keep every load above in flight before anything waits on one of them
+    __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-        if (c + 1 < NCH) load_a(c + 1, a[(c + 1) & 1]);
+        if (c + 1 < NCH) { load_a(c + 1, a[(c + 1) & 1]); __builtin_amdgcn_sched_barrier(0); }
         if constexpr (NORM != SN_NONE) {
             // row sums of squares over this wave's K slice, then over the 8 waves
             float ss[SK_MTS];
@@ -142,22 +147,23 @@ void skinny_kernel(SkinnyP p) {
     }
     if (m >= p.M) return;
     const int n0 = tile * 16 + 4 * g;
+    bf16_t* const optr = p.out_tiled ? p.out + ft_index(m + p.out_row0, n0, p.ldo >> 5) : p.out + (size_t)m * p.ldo + n0;
     if constexpr (EPI == SK_BIAS || EPI == SK_BIAS_SILU) {
         f32x4 o = v[0];
         const bf16x4 bb = load4(p.bias + n0);
 #pragma unroll
         for (int e = 0; e < 4; ++e) { o[e] += bf2f(bb[e]); if (EPI == SK_BIAS_SILU) o[e] = siluf(o[e]); }
-        store4(p.out + (size_t)m * p.ldo + n0, pack4(o));
+        store4(optr, pack4(o));
     } else if constexpr (EPI == SK_RES) {
         f32x4 o = v[0];
         if (p.gate) { const bf16x4 gg = load4(p.gate + n0); for (int e = 0; e < 4; ++e) o[e] *= bf2f(gg[e]); }
         if (p.bias) { const bf16x4 bb = load4(p.bias + n0); for (int e = 0; e < 4; ++e) o[e] += bf2f(bb[e]); }
-        const bf16x4 old = load4(p.out + (size_t)m * p.ldo + n0);
+        const bf16x4 old = load4(optr);
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] += bf2f(old[e]);
-        store4(p.out + (size_t)m * p.ldo + n0, pack4(o));
+        store4(optr, pack4(o));
     } else if constexpr (EPI == SK_GEGLU) {
-        store4(p.out + (size_t)m * p.ldo + n0,
+        store4(optr,
                pack4(gelu_tanh(v[0][0]) * v[1][0], gelu_tanh(v[0][1]) * v[1][1], gelu_tanh(v[0][2]) * v[1][2], gelu_tanh(v[0][3]) * v[1][3]));
     } else if constexpr (EPI == SK_QKV_ROPE) {
         f32x4 o = v[0];
@@ -167,12 +173,12 @@ void skinny_kernel(SkinnyP p) {
             const f32x4 x = o;
             o[0] = x[0] * c0 - x[1] * s0; o[1] = x[1] * c0 + x[0] * s0;
             o[2] = x[2] * c1 - x[3] * s1; o[3] = x[3] * c1 + x[2] * s1;
-            if (n0 < 2048) store4(p.q + (size_t)m * 2048 + n0, pack4(o));
-            else store4(p.k + (size_t)(p.kv_row0 + m) * 256 + (n0 - 2048), pack4(o));
+            if (n0 < 2048) store4(p.q + ft_index(m * 8 + (n0 >> 8), n0 & 255, 8), pack4(o));
+            else store4(p.k + ft_index(p.kv_row0 + m, n0 - 2048, 8), pack4(o));
         } else {
             const int d = n0 - 2304;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) p.vt[(size_t)(d + e) * p.ldvt + p.kv_row0 + m] = f2bf(o[e]);
+            for (int e = 0; e < 4; ++e) p.vt[vt_index(d + e, p.kv_row0 + m, p.ldvt >> 5)] = f2bf(o[e]);
         }
     }
 }
@@ -195,7 +201,8 @@ int launch_inst(const SkinnyP& p, hipStream_t s) {
 int launch_skinny(const SkinnyP& p, int epi, hipStream_t s) {
     if (p.M <= 0 || p.M > 64 || p.N16 <= 0) return 1;
     if (p.K != 1024 && p.K != 2048 && p.K != 4096) return 1;
-    if (p.K32p < p.K / 32 || p.lda < p.K) return 1;
+    if (p.K32p < p.K / 32 || p.lda < p.K || (p.lda & 31)) return 1;
+    if (p.out_tiled && (p.ldo & 31)) return 1;
     const int nch = p.K / (32 * SK_WAVES * SK_CH);
     if (p.norm != SN_NONE && nch != 1) return 1;
     if (p.norm == SN_ADARMS && !p.style) return 1;

@@ -54,6 +54,8 @@ SYMBOLS = {
     "rtvla_graph_launch": (ctypes.c_int, [_P, _P]),
     "rtvla_launch_count": (ctypes.c_int, [_P]),
     "rtvla_time_stage": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P, ctypes.POINTER(ctypes.c_float)]),
+    "rtvla_time_launch": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P,
+                                         ctypes.POINTER(ctypes.c_float), ctypes.c_char_p, ctypes.c_size_t]),
     "rtvla_time_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.POINTER(ctypes.c_float)]),
     "rtvla_pretile_elems": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "rtvla_pretile": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P]),
@@ -160,6 +162,16 @@ class Context:
         ms = ctypes.c_float()
         self.check(self.lib.rtvla_time_stage(self.handle, stage, layer, step, iters, _P(stream), ctypes.byref(ms)))
         return ms.value
+
+    def time_launch(self, stage, layer, step, index, iters, stream):
+        """(mean ms, launch name) of the index-th kernel of a stage; None past the end."""
+        ms = ctypes.c_float()
+        name = ctypes.create_string_buffer(64)
+        rc = self.lib.rtvla_time_launch(self.handle, stage, layer, step, index, iters, _P(stream), ctypes.byref(ms), name, 64)
+        if rc == 1:
+            return None
+        self.check(rc)
+        return ms.value, name.value.decode()
 
     def time_forward(self, iters, stream):
         arr = (ctypes.c_float * iters)()
