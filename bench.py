@@ -1,0 +1,146 @@
+"""Latency benchmark of the Pi0 / Pi05 single-observation forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config headline|c1|c2|c3|c4|c5] [--no-cpu]
+
+A "step" is one forward (vision encoder + prefix pass + 10 flow steps) on synthetic inputs that are
+already resident in HBM.  Prints ONE JSON line: p50 latency (ms) as `value`, the live roofline of the
+dominant kernel, and the CPU oracle timed on the host cores as a reported baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "realtime-vla_amd"))
+
+CONFIGS = {
+    # name: (model, views, prompt_len, chunk, state_tokens, description)
+    "headline": ("pi0", 3, 20, 50, 0, "Pi0, 3 views, 20-token prompt, chunk 50, 10 flow steps"),
+    "c1": ("pi0", 1, 0, 50, 0, "Pi0, 1 view, empty prompt, chunk 50, 10 flow steps"),
+    "c2": ("pi0", 2, 20, 50, 0, "Pi0, 2 views, 20-token prompt, chunk 50, 10 flow steps"),
+    "c3": ("pi0", 3, 0, 63, 0, "Pi0, 3 views, empty prompt, chunk 63, 10 flow steps"),
+    "c4": ("pi05", 3, 20, 50, 32, "Pi05, 3 views, 20 prompt + 32 state tokens, chunk 50, 10 flow steps"),
+    "c5": ("pi0", 3, 200, 50, 0, "Pi0, 3 views, 200-token prompt (968-token prefix), chunk 50, 10 flow steps"),
+}
+MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs one observation on ONE GPU; --gpus %d is not supported "
+              "(see DESIGN.md, 'More than one GPU')" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import synthetic as syn
+    import rtvla_capi as capi
+    capi.load()                                   # no fallback: fail loudly if the HIP library is missing
+    model_name, views, prompt, chunk, state_tokens, desc = CONFIGS[args.config]
+    dev = "cuda:0"
+    seed = 1234
+    if model_name == "pi0":
+        from pi0_infer import Pi0Inference
+        ck = syn.pi0_checkpoint(seed, prompt, device=dev)
+        img, state, noise = syn.observation(seed, views, chunk, device=dev)
+        model = Pi0Inference(ck, views, chunk)
+        run = lambda nz: model.forward(img, state, nz)
+    else:
+        from pi05_infer import Pi05Inference
+        ck = syn.pi05_checkpoint(seed, prompt, device=dev, state_tokens=state_tokens)
+        img, state, noise = syn.observation(seed, views, chunk, device=dev)
+        model = Pi05Inference(ck, views, chunk, discrete_state_input=False)
+        run = lambda nz: model.forward(img, nz)
+    ctx = model._engine.ctx
+    stream = torch.cuda.current_stream().cuda_stream
+    # fresh noise every iteration (BASELINE config 5); drawn up front so the timed region holds only forward()
+    draws = [syn.observation(seed, views, chunk, device=dev, draw=i % 16)[2] for i in range(16)]
+
+    for i in range(args.warmup):
+        run(draws[i % 16])
+    torch.cuda.synchronize()
+    times = []
+    t_all0 = time.perf_counter()
+    for i in range(args.steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run(draws[i % 16])
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    t_all = (time.perf_counter() - t_all0) * 1e3
+    st = sorted(times)
+    p50 = st[len(st) // 2]
+    p99 = st[min(len(st) - 1, int(0.99 * len(st)))]
+
+    # ---- roofline of the dominant kernel, measured live with HIP events on its own stream ----------
+    S_v = 256 * views
+    S_e = S_v + prompt + state_tokens
+    S_d = chunk + (1 if model_name == "pi0" else 0)
+    keys = S_e + S_d
+    # dominant kernel: the Gemma-prefix GeGLU GEMM (gate and up, 2048 -> 16384 each): launch index 4 of a prefix layer
+    geglu_ms, geglu_name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, 4, 20, stream)
+    geglu_flop = 2.0 * 2.0 * S_e * 2048 * 16384
+    mfma = geglu_flop / (geglu_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "prefix GeGLU GEMM (gemm_mfma_kernel, EPI_GEGLU), M=%d K=2048 N=2x16384" % S_e,
+                "achieved": round(mfma, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(mfma / MFMA_PEAK_TFLOPS, 4),
+                "launch_ms": round(geglu_ms, 4), "traffic": None}
+    # the action-expert side: one suffix layer (5 launches) streams 18 D_L-sized weight sets per step
+    layer_ms = ctx.time_stage(capi.STAGE_SUFFIX_LAYER, 3, 0, 20, stream)
+    d_l = 1024 * 2560 + 2048 * 1024 + 3 * 1024 * 4096
+    layer_bytes = 2.0 * d_l + 2.0 * keys * 256 * 2
+    hbm = layer_bytes / (layer_ms * 1e-3) / 1e9
+    roofline_hbm = {"bound": "hbm", "kernel": "one action-expert layer (qkv, attention, o, geglu, down)",
+                    "achieved": round(hbm, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hbm / HBM_PEAK_GBS, 4),
+                    "launch_ms": round(layer_ms, 4), "traffic": None}
+    # whole-forward roofline fraction: (F_vis + F_pre) / P_mfma + B_dec / BW  over the measured p50
+    v_l = 1152 * 3456 + 1152 * 1152 + 2 * 1152 * 4304
+    e_l = 2048 * 2560 + 2048 * 2048 + 3 * 2048 * 16384
+    f_vis = 2.0 * S_v * (588 * 1152 + 27 * v_l + 1152 * 2048) + 27 * views * 16 * 4 * 256 * 256 * 72
+    f_pre = 2.0 * S_e * (17 * e_l + 2048 * 512) + 17 * 8 * 4 * S_e * S_e * 256
+    x_bytes = (32 * 1024 + 1024 * 1024 + 1024 * 32) if model_name == "pi0" else (32 * 1024 + 1024 * 32)
+    b_dec = 10 * (2.0 * (18 * d_l + x_bytes) + 18 * 2 * keys * 256 * 2 + (37 * 3072 * 2 if model_name == "pi05" else 0))
+    ideal_ms = ((f_vis + f_pre) / (MFMA_PEAK_TFLOPS * 1e12) + b_dec / (HBM_PEAK_GBS * 1e9)) * 1e3
+
+    result = {
+        "metric": "p50 ms per Pi0 forward (3 views, chunk 50, 10 steps); % roofline",
+        "value": round(p50, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(t_all / args.steps, 4), "p99_ms": round(p99, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": desc, "config_id": args.config, "S_v": S_v, "S_e": S_e, "S_d": S_d, "keys": keys,
+                   "graph_launches": model._engine.graph_launches, "weights": "seeded N(0, 0.02^2) bf16, norms = 1"},
+        "roofline": roofline, "roofline_hbm": roofline_hbm,
+        "forward_roofline_frac": round(ideal_ms / p50, 4), "forward_ideal_ms": round(ideal_ms, 4),
+        "reference_published": {"value_ms": 39.2, "hardware": "RTX 4090, Triton", "source": "README.md:18"} if args.config == "headline" else None,
+    }
+
+    # ---- CPU baseline: the oracle (a port of the reference math) on the host cores, one forward ----
+    if not args.no_cpu:
+        from oracle import pi0 as o0, pi05 as o5          # the checker, timed as a baseline only
+        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or os.cpu_count()
+        torch.set_num_threads(cores)
+        ckc = {k: v.cpu() for k, v in ck.items()}
+        t0 = time.perf_counter()
+        if model_name == "pi0":
+            ref = o0.forward(ckc, img.cpu(), state.cpu(), draws[0].cpu())
+        else:
+            ref = o5.forward(ckc, img.cpu(), draws[0].cpu())
+        cpu_ms = (time.perf_counter() - t0) * 1e3
+        out = run(draws[0]).float().cpu()
+        result["cpu_baseline"] = {"value": round(cpu_ms, 1), "unit": "ms", "cores": cores, "kind": "port",
+                                  "sample": "one forward of the same workload (no warm-up), PyTorch CPU eager oracle"}
+        result["action_mae_vs_oracle"] = round((out - ref).abs().mean().item(), 5)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -66,6 +66,7 @@ class Engine:
         side.wait_stream(torch.cuda.current_stream(self.device))
         self.ctx.graph_capture(side.cuda_stream)
         side.synchronize()
+        self.graph_launches = self.ctx.launch_count()      # kernel nodes in the captured graph
 
     def replay(self):
         self.ctx.graph_launch(torch.cuda.current_stream(self.device).cuda_stream)
@@ -97,3 +98,10 @@ def untile_vt(flat, d, keys_pad):
     register j holding key 32*tile + 4 g + (j & 3) + 16 (j >> 2)."""
     t = flat.reshape(-1)[: d * keys_pad].view(d // 16, keys_pad // 32, 4, 16, 2, 4)     # [dt][kt][g][r][hi][lo]
     return t.permute(0, 3, 1, 4, 2, 5).reshape(d, keys_pad)
+
+
+def tile_vt(mat):
+    """Inverse of untile_vt: row-major [d][keys_pad] -> flat transposed-V tile layout."""
+    d, keys_pad = mat.shape
+    t = mat.reshape(d // 16, 16, keys_pad // 32, 2, 4, 4)                                # [dt][r][kt][hi][g][lo]
+    return t.permute(0, 2, 4, 1, 3, 5).reshape(-1)

@@ -1,0 +1,101 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports every symbol the
+header declares, validates dimensions and bindings, and reports errors as status codes."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import rtvla_capi as capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(capi.LIB_PATH):
+        import build
+        build.build(force=True)
+    return capi.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    header = open(os.path.join(ROOT, "include", "rtvla.h")).read()
+    declared = set(re.findall(r"\b(rtvla_[a-z_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    assert declared == set(capi.SYMBOLS), "binding table and header differ: %s" % (declared ^ set(capi.SYMBOLS))
+    for name in declared:
+        assert hasattr(lib, name)
+    assert lib.rtvla_version() >= 1
+
+
+def test_create_validates_dimensions(lib):
+    for bad in [(capi.PI0, 0, 0, 50), (capi.PI0, 5, 0, 50), (capi.PI0, 1, -1, 50), (capi.PI0, 1, 0, 0), (2, 1, 0, 50)]:
+        with pytest.raises(capi.RtvlaError):
+            capi.Context(*bad)
+    with pytest.raises(capi.RtvlaError) as e:
+        capi.Context(capi.PI0, 1, 0, 64)          # 65 suffix rows do not fit the 64-row suffix tile
+    assert e.value.code == 7
+    capi.Context(capi.PI0, 1, 0, 63).close()
+    capi.Context(capi.PI05, 3, 52, 64).close()
+
+
+def test_tensor_table_matches_the_reference_layout(lib):
+    c = capi.Context(capi.PI0, 3, 20, 50)
+    t = {n: (e, s, w) for n, e, s, w, _ in c.tensors()}
+    assert t["vision_patch_embedding_w"] == (2, (14, 14, 3, 1152), True)
+    assert t["encoder_ffn_gate_w"] == (2, (18, 2048, 16384), True)
+    assert t["decoder_action_fused_time_biases"] == (2, (10, 1024), True)
+    assert t["language_embeds"] == (2, (20, 2048), True)
+    assert t["diffusion_noise"] == (2, (50, 32), False)
+    assert t["encoder_rope_weights"] == (2, (788, 256), False)
+    assert t["decoder_rope_weights"] == (2, (51, 256), False)
+    assert len([n for n, v in t.items() if v[2]]) == 38      # pi0_infer.py:1245-1287 lists 38 weights
+    c5 = capi.Context(capi.PI05, 3, 52, 50)
+    t5 = {n: (e, s, w) for n, e, s, w, _ in c5.tensors()}
+    assert t5["valid_encoder_len"] == (4, (1,), False)
+    assert t5["decoder_pre_attn_norm_mod_w"] == (2, (18, 1024, 3072), True)
+    assert t5["decoder_rope_weights"] == (2, (50, 256), False)
+    assert "observation_state_normalized" not in t5 and "decoder_state_in_proj_w" not in t5
+
+
+def test_bind_errors_are_status_codes(lib):
+    c = capi.Context(capi.PI0, 1, 0, 50)
+    with pytest.raises(capi.RtvlaError) as e:
+        c.bind("no_such_tensor", 256, 16)
+    assert e.value.code == capi.ERR_NAME and "no_such_tensor" in str(e.value)
+    with pytest.raises(capi.RtvlaError) as e:
+        c.bind("diffusion_noise", 256, 50 * 32 * 2 + 2)
+    assert e.value.code == capi.ERR_SIZE
+    with pytest.raises(capi.RtvlaError):
+        c.bind("diffusion_noise", 0, 50 * 32 * 2)           # null pointer
+    with pytest.raises(capi.RtvlaError):
+        c.bind("diffusion_noise", 257, 50 * 32 * 2)         # misaligned
+    c.bind("language_embeds", 0, 0)                          # an empty prompt binds a null, zero-byte tensor
+
+
+def test_calls_out_of_order_are_rejected(lib):
+    c = capi.Context(capi.PI0, 1, 0, 50)
+    for fn in (c.prepare, c.forward, c.graph_capture):
+        with pytest.raises(capi.RtvlaError) as e:
+            fn(0)
+        assert e.value.code in (4, 5)
+    with pytest.raises(capi.RtvlaError):
+        c.graph_launch(0)
+    with pytest.raises(capi.RtvlaError):
+        c.bind_workspace(256, 1024)                          # too small
+    assert lib.rtvla_forward(None, None) == 1 and lib.rtvla_destroy(None) == 1
+
+
+def test_workspace_layout(lib):
+    small = capi.Context(capi.PI0, 1, 0, 50, vision_layers=2, llm_layers=2)
+    big = capi.Context(capi.PI0, 3, 200, 50)
+    assert 0 < small.workspace_bytes() < big.workspace_bytes() < 8 << 30
+    bufs = {n: (off, rows, cols, ld, e) for n, off, rows, cols, ld, e in big.buffers()}
+    assert bufs["encoder_x"][1:4] == (968, 2048, 2048)
+    assert bufs["vision_hidden"][2:4] == (4304, 4352)        # K padded to the 128-wide stage pair
+    assert bufs["splitk_partial"][4] == 4
+    offs = sorted((v[0], v[0] + v[1] * v[3] * v[4]) for v in bufs.values())
+    assert all(a[1] <= b[0] for a, b in zip(offs, offs[1:])), "workspace regions overlap"
+    assert all(v[0] % 256 == 0 for v in bufs.values())
+    assert lib.rtvla_pretile_elems(588, 1152) == 72 * 20 * 512
