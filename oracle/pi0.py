@@ -93,6 +93,8 @@ def transformer_decoder(w, ks, vs, state, noise, rnd, taps=None, num_steps=10):
         u = rnd(ops.silu(f32(w["decoder_action_fused_time_biases"][t % 10]) + gemm(noise, w["decoder_action_fused_in_proj_w"])))
         xa = rnd(f32(w["decoder_action_mlp_b"]) + gemm(u, w["decoder_action_mlp_w"]))
         x = torch.cat([s, xa], dim=0)
+        if taps is not None:
+            taps["decoder_in/%d" % t] = x.clone()
         for i in range(layers):
             f = rnd(ops.rms_factor(x))
             acc = gemm(x, w["decoder_attn_qkv_w"][i]) * f            # scale applied to the fp32 accumulator (:1005)

@@ -46,6 +46,8 @@ def transformer_decoder(w, ks, vs, noise, valid_len, rnd, taps=None, num_steps=1
     noise = f32(noise)
     for t in range(num_steps):
         x = rnd(f32(w["decoder_action_in_proj_b"]) + gemm(noise, w["decoder_action_in_proj_w"]))
+        if taps is not None:
+            taps["decoder_in/%d" % t] = x.clone()
         for i in range(layers):
             n, gate = adarms(x, st_attn[t][i], rnd)
             acc = gemm(n, w["decoder_attn_qkv_w"][i])

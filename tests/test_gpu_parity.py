@@ -1,0 +1,310 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle and the golden fixtures.
+
+Tolerances are the ones the task states for this floating-point path: action MAE <= 1e-2 against
+the bf16-boundary oracle, per-layer relative L2 <= 2e-2.  "Per layer" is measured layer-locally:
+each stage is fed the oracle's input for that layer (teacher forcing) so that the bf16 drift two
+independent pipelines accumulate over 45 layers (3e-2 between the oracle's own bf16 and fp32
+variants) is not charged to any single kernel.  Free-running drift is printed for the record.
+"""
+import os
+
+import pytest
+import torch
+
+import synthetic as syn
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+MAE_TOL = 1e-2
+LAYER_TOL = 2e-2
+
+
+def rel(a, b):
+    a, b = a.float().cpu(), b.float().cpu()
+    return ((a - b).norm() / (b.norm() + 1e-30)).item()
+
+
+def bf(x, dev="cuda"):
+    return x.to(torch.bfloat16).to(dev)
+
+
+class Case:
+    """One model instance + its oracle run with taps."""
+
+    def __init__(self, model, seed, views, prompt, chunk, vision_layers=27, llm_layers=18, state_tokens=0, max_prompt=None):
+        import rtvla_capi as capi
+        from oracle import pi0 as o0, pi05 as o5, ops
+        self.capi, self.ops = capi, ops
+        self.model_name, self.views, self.chunk = model, views, chunk
+        self.VL, self.LL = vision_layers, llm_layers
+        dev = "cuda:0"
+        if model == "pi0":
+            from pi0_infer import Pi0Inference
+            self.ck = syn.pi0_checkpoint(seed, prompt, dev, vision_layers, llm_layers)
+            self.img, self.state, self.noise = syn.observation(seed, views, chunk, dev)
+            self.m = Pi0Inference(self.ck, views, chunk)
+            self.S_e = 256 * views + prompt
+            self.S_d = chunk + 1
+            self.valid = self.S_e
+        else:
+            from pi05_infer import Pi05Inference
+            self.ck = syn.pi05_checkpoint(seed, prompt, dev, vision_layers, llm_layers, state_tokens=state_tokens)
+            self.img, self.state, self.noise = syn.observation(seed, views, chunk, dev)
+            plen = prompt + state_tokens
+            if max_prompt is not None and max_prompt != plen:
+                # allocate a longer prefix than the prompt: pad the checkpoint's prompt, then shorten it per call
+                pad = torch.zeros(max_prompt - plen, 2048, dtype=torch.bfloat16, device=dev)
+                ck2 = dict(self.ck); ck2["language_embeds"] = torch.cat([self.ck["language_embeds"], pad])
+                self.m = Pi05Inference(ck2, views, chunk, discrete_state_input=False)
+                self.m.weights["language_embeds"] = self.ck["language_embeds"].clone()
+            else:
+                self.m = Pi05Inference(self.ck, views, chunk, discrete_state_input=False)
+            self.S_e = 256 * views + (max_prompt if max_prompt is not None else plen)
+            self.S_d = chunk
+            self.valid = 256 * views + plen
+        self.ckc = {k: v.cpu() for k, v in self.ck.items()}
+        self.taps = {}
+        if model == "pi0":
+            self.ref = o0.forward(self.ckc, self.img.cpu(), self.state.cpu(), self.noise.cpu(), taps=self.taps)
+        else:
+            self.ref = o5.forward(self.ckc, self.img.cpu(), self.noise.cpu(), max_prompt_len=max_prompt, taps=self.taps)
+        self.e, self.B = self.m._engine, self.m.buffers
+        self.keys_pad = self.B["encoder_Vt"].shape[1]
+
+    # ---- input staging (what forward() does before the replay) ----
+    def stage_inputs(self):
+        if self.model_name == "pi0":
+            self.B["observation_images_normalized"].copy_(self.img)
+            self.B["observation_state_normalized"].copy_(self.state)
+            self.B["diffusion_noise"].copy_(self.noise)
+        else:
+            self.m.stage_inputs(self.img, self.noise)
+
+    def forward(self):
+        if self.model_name == "pi0":
+            return self.m.forward(self.img, self.state, self.noise)
+        return self.m.forward(self.img, self.noise)
+
+    def run(self, stage, layer=0, step=0):
+        self.e.run_stage(stage, layer, step)
+        torch.cuda.synchronize()
+
+    # ---- buffer access in the library's layouts ----
+    def dec_x(self):
+        from _engine import untile_ft
+        return untile_ft(self.B["decoder_x"], 64, 1024)[: self.S_d]
+
+    def set_dec_x(self, x):
+        from _engine import tile_ft
+        full = torch.zeros(64, 1024, dtype=torch.bfloat16, device="cuda")
+        full[: self.S_d] = bf(x)
+        self.B["decoder_x"].reshape(-1).copy_(tile_ft(full))
+
+    def cache(self, i):
+        from _engine import untile_ft, untile_vt
+        K = untile_ft(self.B["encoder_K"].reshape(self.LL, -1)[i], self.keys_pad, 256)
+        V = untile_vt(self.B["encoder_Vt"].reshape(self.LL, -1)[i], 256, self.keys_pad).t()
+        return K, V
+
+    def set_cache_prefix(self, i, k, v):
+        from _engine import tile_ft, tile_vt
+        K, V = self.cache(i)
+        K = K.clone(); V = V.clone()
+        K[: self.S_e] = bf(k); V[: self.S_e] = bf(v)
+        self.B["encoder_K"].reshape(self.LL, -1)[i].copy_(tile_ft(K))
+        self.B["encoder_Vt"].reshape(self.LL, -1)[i].copy_(tile_vt(V.t().contiguous()))
+
+    # ---- the checks ----
+    def free_running(self):
+        """Whole forward stage by stage; returns the drift per tap and the final MAE."""
+        c, t = self.capi, self.taps
+        self.stage_inputs()
+        drift = {}
+        self.run(c.STAGE_VISION_EMBED)
+        drift["vision_embed"] = rel(self.B["vision_x"], t["vision_embed"])
+        for i in range(self.VL):
+            self.run(c.STAGE_VISION_LAYER, i)
+            drift["vision_x/%d" % i] = rel(self.B["vision_x"], t["vision_x/%d" % i])
+        self.run(c.STAGE_PROJECT)
+        drift["encoder_x0"] = rel(self.B["encoder_x"][: self.valid], t["encoder_x0"][: self.valid])
+        for i in range(self.LL):
+            self.run(c.STAGE_PREFIX_LAYER, i)
+            K, V = self.cache(i)
+            drift["encoder_K/%d" % i] = rel(K[: self.valid], t["encoder_K/%d" % i][: self.valid])
+            drift["encoder_V/%d" % i] = rel(V[: self.valid], t["encoder_V/%d" % i][: self.valid])
+        self.run(c.STAGE_SUFFIX_INIT)
+        for s in range(10):
+            self.run(c.STAGE_SUFFIX_STEP_BEGIN, 0, s)
+            for i in range(self.LL):
+                self.run(c.STAGE_SUFFIX_LAYER, i, s)
+            drift["decoder_x/%d" % s] = rel(self.dec_x(), t["decoder_x/%d/%d" % (s, self.LL - 1)])
+            self.run(c.STAGE_SUFFIX_STEP_END, 0, s)
+            drift["noise/%d" % s] = rel(self.B["diffusion_noise"], t["noise/%d" % s])
+        out = self.B["diffusion_noise"].float().cpu().clone()
+        return drift, out
+
+    def teacher_forced(self, steps=(0, 9)):
+        """Every layer fed the oracle's input; returns the layer-local relative L2 per layer."""
+        c, t, ops, w = self.capi, self.taps, self.ops, self.ckc
+        errs = {}
+        self.stage_inputs()
+        self.run(c.STAGE_VISION_EMBED)
+        errs["vision_embed"] = rel(self.B["vision_x"], t["vision_embed"])
+        for i in range(self.VL):
+            x = t["vision_embed"] if i == 0 else t["vision_x/%d" % (i - 1)]
+            self.B["vision_x"].copy_(bf(x))
+            self.B["vision_x_norm"].copy_(bf(ops.layer_norm(x, w["vision_pre_attn_norm_w"][i], w["vision_pre_attn_norm_b"][i])))
+            self.run(c.STAGE_VISION_LAYER, i)
+            errs["vision_layer/%d" % i] = rel(self.B["vision_x"], t["vision_x/%d" % i])
+        x = t["vision_x/%d" % (self.VL - 1)]
+        self.B["vision_x_norm"].copy_(bf(ops.layer_norm(x, w["vision_final_norm_w"], w["vision_final_norm_b"])))
+        self.run(c.STAGE_PROJECT)
+        errs["project"] = rel(self.B["encoder_x"][: self.valid], t["encoder_x0"][: self.valid])
+        for i in range(self.LL):
+            x = t["encoder_x0"] if i == 0 else t["encoder_x/%d" % (i - 1)]
+            self.B["encoder_x"].copy_(bf(x))
+            self.B["encoder_x_norm"].copy_(bf(x * ops.rms_factor(x)))
+            self.run(c.STAGE_PREFIX_LAYER, i)
+            K, V = self.cache(i)
+            errs["prefix_K/%d" % i] = rel(K[: self.valid], t["encoder_K/%d" % i][: self.valid])
+            errs["prefix_V/%d" % i] = rel(V[: self.valid], t["encoder_V/%d" % i][: self.valid])
+            if i != self.LL - 1:
+                errs["prefix_layer/%d" % i] = rel(self.B["encoder_x"][: self.valid], t["encoder_x/%d" % i][: self.valid])
+        for i in range(self.LL):
+            self.set_cache_prefix(i, t["encoder_K/%d" % i], t["encoder_V/%d" % i])
+        self.run(c.STAGE_SUFFIX_INIT)
+        for s in steps:
+            noise_in = self.noise.float().cpu() if s == 0 else t["noise/%d" % (s - 1)]
+            self.B["diffusion_noise"].copy_(bf(noise_in))
+            self.run(c.STAGE_SUFFIX_STEP_BEGIN, 0, s)
+            errs["suffix_in/%d" % s] = rel(self.dec_x(), t["decoder_in/%d" % s])
+            for i in range(self.LL):
+                x = t["decoder_in/%d" % s] if i == 0 else t["decoder_x/%d/%d" % (s, i - 1)]
+                self.set_dec_x(x)
+                self.run(c.STAGE_SUFFIX_LAYER, i, s)
+                errs["suffix_layer/%d/%d" % (s, i)] = rel(self.dec_x(), t["decoder_x/%d/%d" % (s, i)])
+            self.set_dec_x(t["decoder_x/%d/%d" % (s, self.LL - 1)])
+            self.B["diffusion_noise"].copy_(bf(noise_in))
+            self.run(c.STAGE_SUFFIX_STEP_END, 0, s)
+            errs["euler/%d" % s] = (self.B["diffusion_noise"].float().cpu() - t["noise/%d" % s]).abs().mean().item()
+        return errs
+
+
+def check_case(case, gold_key=None, gold_file="golden_small.pt"):
+    drift, staged = case.free_running()
+    mae = (staged - case.ref).abs().mean().item()
+    worst = max(drift, key=drift.get)
+    print("\n[%s] free-running: action MAE %.5f, largest cumulative rel-L2 %.4f at %s" % (gold_key, mae, drift[worst], worst))
+    assert torch.isfinite(staged).all()
+    assert mae <= MAE_TOL
+    per_dim = (staged - case.ref).abs().mean(0)
+    assert per_dim.max().item() <= 3 * MAE_TOL          # per-dimension MAE, the second statistic of test.py:282-287
+    out = case.forward().float().cpu()                    # the captured graph, same inputs
+    assert torch.equal(out, staged), "graph replay differs from the staged eager run"
+    assert torch.equal(case.forward().float().cpu(), out), "two replays differ"
+    if gold_key:
+        g = torch.load(os.path.join(GOLD, gold_file), weights_only=True)
+        assert (out - g[gold_key + "/actions"].float()).abs().mean().item() <= MAE_TOL
+        assert (out - g[gold_key + "/actions_fp32"]).abs().mean().item() <= MAE_TOL
+        # the oracle re-run on this host's CPU agrees with the committed vector up to the BLAS summation order
+        assert (case.ref - g[gold_key + "/actions"].float()).abs().mean().item() <= 0.5 * MAE_TOL
+    errs = case.teacher_forced()
+    layer = {k: v for k, v in errs.items() if not k.startswith("euler")}
+    worst = max(layer, key=layer.get)
+    print("[%s] teacher-forced: worst layer-local rel-L2 %.5f at %s; Euler MAE %.5f" %
+          (gold_key, layer[worst], worst, max(v for k, v in errs.items() if k.startswith("euler"))))
+    assert layer[worst] <= LAYER_TOL, (worst, layer[worst])
+    assert all(v <= MAE_TOL for k, v in errs.items() if k.startswith("euler"))
+    return mae
+
+
+def test_pi0_reduced_depth_staged_and_graph():
+    check_case(Case("pi0", 7, 1, 4, 10, 2, 2), "pi0_small")
+
+
+def test_pi0_empty_prompt_max_chunk():
+    check_case(Case("pi0", 8, 1, 0, 63, 1, 2), "pi0_small_noprompt_c63")
+
+
+def test_pi05_reduced_depth_with_padded_prefix():
+    check_case(Case("pi05", 9, 1, 4, 10, 2, 2, state_tokens=3, max_prompt=12), "pi05_small")
+
+
+def test_pi0_two_views_ragged_prefix():
+    check_case(Case("pi0", 21, 2, 7, 17, 1, 2))
+
+
+@pytest.mark.parametrize("name,spec", [
+    ("c1", ("pi0", 1234, 1, 0, 50)),
+    ("c2", ("pi0", 1234, 2, 20, 50)),
+    ("c3", ("pi0", 1234, 3, 0, 63)),
+])
+def test_pi0_full_size_configs(name, spec):
+    check_case(Case(*spec), name, "golden_full.pt")
+
+
+def test_pi05_full_size_c4():
+    check_case(Case("pi05", 1234, 3, 20, 50, state_tokens=32), "c4", "golden_full.pt")
+
+
+def test_c5_prefix_stress_sustained_replay():
+    """968-token prefix (1019 keys): 100 replays with fresh noise; every 25th checked against eager."""
+    from pi0_infer import Pi0Inference
+    from oracle import pi0 as o0
+    ck = syn.pi0_checkpoint(1234, 200, "cuda:0")
+    img, state, noise = syn.observation(1234, 3, 50, "cuda:0")
+    m = Pi0Inference(ck, 3, 50)
+    ref = o0.forward({k: v.cpu() for k, v in ck.items()}, img.cpu(), state.cpu(), noise.cpu())
+    out = m.forward(img, state, noise).float().cpu()
+    assert (out - ref).abs().mean().item() <= MAE_TOL
+    for it in range(100):
+        nz = syn.observation(1234, 3, 50, "cuda:0", draw=it)[2]
+        got = m.forward(img, state, nz).clone()
+        if it % 25 == 0:
+            m.buffers["diffusion_noise"].copy_(nz)
+            m.record_run()
+            torch.cuda.synchronize()
+            assert torch.equal(got, m.buffers["diffusion_noise"])
+        assert torch.isfinite(got.float()).all()
+    assert torch.equal(m.forward(img, state, noise).float().cpu(), out)
+
+
+def test_zero_output_projection_returns_the_noise_bit_exactly():
+    from pi0_infer import Pi0Inference
+    ck = syn.pi0_checkpoint(3, 2, "cuda:0", 1, 2)
+    ck["decoder_action_fused_out_proj_w"].zero_(); ck["decoder_action_fused_out_proj_b"].zero_()
+    img, state, noise = syn.observation(3, 1, 12, "cuda:0")
+    out = Pi0Inference(ck, 1, 12).forward(img, state, noise)
+    assert torch.equal(out, noise)
+
+
+def test_forward_contract_dtypes_devices_and_aliasing():
+    from pi0_infer import Pi0Inference
+    ck = syn.pi0_checkpoint(4, 3, "cuda:0", 1, 2)
+    img, state, noise = syn.observation(4, 1, 10, "cuda:0")
+    m = Pi0Inference({k: v.cpu() for k, v in ck.items()}, 1, 10)        # CPU checkpoint tensors are copied in
+    a = m.forward(img, state, noise).clone()
+    b = m.forward(img.float().cpu(), state.float().cpu(), noise.float())    # fp32 / CPU inputs, test.py:188-190
+    assert b.dtype == torch.bfloat16 and b.shape == (10, 32) and b.is_cuda
+    assert torch.equal(a, b)
+    assert b.data_ptr() == m.buffers["diffusion_noise"].data_ptr()        # the live internal buffer, pi0_infer.py:1361
+    assert m.prompt_len == 3 and m.num_views == 1 and m.chunk_size == 10
+    assert set(ck) <= set(m.weights)
+
+
+def test_constructor_errors_match_the_reference():
+    from pi0_infer import Pi0Inference
+    ck = syn.pi0_checkpoint(4, 1, "cuda:0", 1, 1)
+    no_prompt = {k: v for k, v in ck.items() if k != "language_embeds"}
+    with pytest.raises(KeyError):
+        Pi0Inference(no_prompt, 1, 10)
+    with pytest.raises(KeyError):
+        Pi0Inference(dict(ck, not_a_weight=torch.zeros(1)), 1, 10)
+    with pytest.raises(RuntimeError):
+        Pi0Inference(dict(ck, vision_final_norm_w=torch.zeros(7)), 1, 10)
+    with pytest.raises(RuntimeError):
+        Pi0Inference(ck, 1, 64)                                            # 65 suffix rows exceed the 64-row tile
+    m = Pi0Inference(ck, 1, 10)
+    with pytest.raises(RuntimeError):
+        m.forward(torch.zeros(2, 224, 224, 3), torch.zeros(32), torch.zeros(10, 32))
