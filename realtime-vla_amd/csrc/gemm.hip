@@ -57,9 +57,12 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    uint4 areg[AIT];
+    bf16x8 areg[AIT];
     bf16x8 breg0[NT][2], breg1[NT][2];
 
+    // LDS stage layout: fragment (row tile i, k half kk) is 1 KB, lane (g, r) at slot (r ^ 8 kk) + 16 g.
+    // The xor spreads the 64 lanes of a staging write (8 rows x 8 chunks) over all banks; a
+    // fragment read still touches every bank exactly once.
     auto load_a = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < AIT; ++it) {
@@ -67,16 +70,16 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
             const int c = min(it * NTH + tid, A_CHUNKS - 1);
             const int row = c >> 3, kc = c & 7;
             const int gr = min(m0 + row, p.a_rows - 1);
-            areg[it] = *(const uint4*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
+            areg[it] = *(const bf16x8*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
         }
     };
     auto store_a = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < AIT; ++it) {
             const int c = min(it * NTH + tid, A_CHUNKS - 1);      // duplicates write identical data
-            const int row = c >> 3, kc = c & 7;
-            const int off = ((((row >> 4) * 2 + (kc >> 2)) * 64) + (row & 15) + 16 * (kc & 3)) * 8;
-            *(uint4*)(lds + buf * STAGE_ELEMS + off) = areg[it];
+            const int row = c >> 3, kc = c & 7, kk = kc >> 2;
+            const int off = ((((row >> 4) * 2 + kk) * 64) + ((row & 15) ^ (kk << 3)) + 16 * (kc & 3)) * 8;
+            *(bf16x8*)(lds + buf * STAGE_ELEMS + off) = areg[it];
         }
     };
     auto load_b = [&](int s, bf16x8 (&br)[NT][2]) __attribute__((always_inline)) {
@@ -86,14 +89,15 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
             for (int kk = 0; kk < 2; ++kk)
                 br[j][kk] = *(const bf16x8*)(bptr[j] + (size_t)(s * 2 + kk) * 512);
     };
+    const int lane_off[2] = {(r + 16 * g) * 8, ((r ^ 8) + 16 * g) * 8};
     auto compute = [&](int buf, bf16x8 (&br)[NT][2]) __attribute__((always_inline)) {
-        const bf16_t* base = lds + buf * STAGE_ELEMS + lane * 8;
+        const bf16_t* base = lds + buf * STAGE_ELEMS;
         // all A fragments of the stage are requested from LDS before the first MFMA waits on one
         bf16x8 af[2][MT];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-            for (int i = 0; i < MT; ++i) af[kk][i] = *(const bf16x8*)(base + (i * 2 + kk) * 512);
+            for (int i = 0; i < MT; ++i) af[kk][i] = *(const bf16x8*)(base + (i * 2 + kk) * 512 + lane_off[kk]);
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
@@ -112,23 +116,25 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         for (int t = 0; t < PRE; ++t) __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
     };
 
-    // stages come in pairs (the host guarantees an even count per split) so that the two register
-    // sets alternate without a runtime index; the loop body is branch free: the last round's
-    // prefetch re-reads a valid stage instead of being skipped
-    if (s_begin < s_end) {
+    // K loop: the loads of stage s+1 fly under the MFMAs of stage s (register-staged A, weights in
+    // a second register set); two stages per trip so the sets alternate without a runtime index and
+    // the body has a single exit.  Past the end the prefetch re-reads the last stage instead of
+    // branching around the loads.
+    const int n_st = s_end - s_begin;
+    if (n_st > 0) {
+        const int last = s_end - 1;
         load_a(s_begin);
         load_b(s_begin, breg0);
         store_a(0);
         __syncthreads();
-        for (int s = s_begin; s < s_end; s += 2) {
+        for (int s = s_begin; s < s_end; s += 2) {          // the host guarantees an even stage count per split
             load_a(s + 1); load_b(s + 1, breg1);
-            __builtin_amdgcn_sched_barrier(0);           // next stage's loads fly under this stage's MFMAs
+            __builtin_amdgcn_sched_barrier(0);
             compute(0, breg0);
             __builtin_amdgcn_sched_barrier(0);
             store_a(1);
             __syncthreads();
-            const int s2 = min(s + 2, s_end - 2);
-            load_a(s2); load_b(s2, breg0);
+            load_a(min(s + 2, last)); load_b(min(s + 2, last), breg0);
             __builtin_amdgcn_sched_barrier(0);
             compute(1, breg1);
             __builtin_amdgcn_sched_barrier(0);

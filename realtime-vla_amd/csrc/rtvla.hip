@@ -100,31 +100,36 @@ namespace {
 constexpr int PATCH_LD = 640;      // 588 patch features padded to a multiple of 64
 constexpr int VHID_LD = 4352;      // 4304 padded to a multiple of 64
 
-// Pick block tile and split-K factor from a coarse cost model: workgroups run in rounds of
-// 256 (one per CU); a workgroup's time is proportional to its valid row tiles x K stages plus a
-// fixed prologue/epilogue; split-K adds the fp32 partial traffic.
+// Pick block tile and split-K factor from a cost model fitted to measurements on MI355X: a workgroup
+// is limited either by its MFMA work or by what one CU can pull from L2 (about 30 GB/s per CU with
+// every CU busy - the L1 miss queue bounds bytes in flight); workgroups run in rounds of 256 (one per
+// CU); every launch pays a fixed ramp; split-K adds the fp32 partial write and read.
 TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable) {
-    static const int tiles[] = {TILE_256x256, TILE_208x256, TILE_128x256, TILE_64x256};
+    static const int tiles[] = {TILE_208x256, TILE_128x256, TILE_64x256};
     static const int splits[] = {1, 2, 3, 4, 6, 8};
     if (const char* e = getenv("RTVLA_FORCE_TILE")) {
         TileChoice c{atoi(e), 1};
         if (const char* s = getenv("RTVLA_FORCE_SPLIT")) if (splittable) c.nsplit = atoi(s);
         return c;
     }
+    const double cu_bw = 30.0e3;           // bytes per microsecond per CU
     double best = 1e30; TileChoice bc{TILE_128x256, 1};
     for (int tile : tiles) {
         const int bm = gemm_tile_bm(tile);
-        const int bn16 = gemm_tile_bn(tile) / 16 / (dual ? 2 : 1);
+        const int bn = gemm_tile_bn(tile);
+        const int bn16 = bn / 16 / (dual ? 2 : 1);
         const int mb = (M + bm - 1) / bm, nb = (ncols16 + bn16 - 1) / bn16;
-        const int mt = (std::min(M, bm) + 15) / 16;
+        const int mt = bm / 16;
         for (int sp : splits) {
             if (sp > 1 && !splittable) break;
             const int sps = (stages + sp - 1) / sp;
             if ((sp - 1) * sps >= stages || (sps & 1)) continue;
             const int blocks = mb * nb * sp;
             const int rounds = (blocks + 255) / 256;
-            double t = rounds * (mt * (sps + 1.0) * 4.0 * 2 * 16 / 2400.0 + 1.5);       // us: MFMA cycles at 2.4 GHz + fixed
-            if (splittable) t += (double)sp * M * ncols16 * 16 * 8.0 / 3.0e6;         // fp32 partial write + read at ~3 TB/s
+            const double mfma_us = mt * sps * 4.0 * 2 * 16 / 2400.0;
+            const double bytes = (double)(std::min(M, bm) + bn) * sps * 64 * 2 + (splittable ? (double)std::min(M, bm) * bn * 4 : 0.0);
+            double t = rounds * std::max(mfma_us, bytes / cu_bw) + 5.0;
+            if (splittable) t += (double)sp * M * ncols16 * 16 * 4.0 / 4.0e6;          // the reduce pass reads the partials at ~4 TB/s
             if (t < best) { best = t; bc = TileChoice{tile, sp}; }
         }
     }
