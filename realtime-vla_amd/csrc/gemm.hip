@@ -14,8 +14,10 @@ namespace {
 
 template <int EPI> struct EpiTraits { static constexpr bool dual = (EPI == EPI_GEGLU); };
 
+// tiles of at most 128 rows are compiled to fit two workgroups per CU (<= 256 registers per lane) so
+// that one workgroup's MFMAs run under the other's memory latency
 template <int WN, int MT, int NT, int EPI>
-__global__ __launch_bounds__(WN * 64) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(WN * 64, (MT <= 8 ? 2 : 1))
 void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int stages_per_split) {
     constexpr int NTH = WN * 64;
     constexpr int BM = MT * 16;
@@ -47,10 +49,12 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         const int t = (n_blk * WN + wn) * HALF + (j % HALF);
         tile_of[j] = t;
         const bf16_t* base = (EpiTraits<EPI>::dual && j >= HALF) ? p.B1 : p.B0;
-        const int tc = min(t, p.N16 - 1);
-        bptr[j] = base + (size_t)tc * p.K32p * 512 + lane * 8;
+        const int G = p.bgroup;
+        const int tc = min(t, ((p.N16 + G - 1) / G) * G - 1);
+        bptr[j] = base + ((size_t)(tc / G) * p.K32p * G + (tc % G)) * 512 + lane * 8;
     }
 
+    const size_t bstep = (size_t)p.bgroup * 512;          // distance between consecutive k32 blocks of one column tile
     f32x4 acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
@@ -87,7 +91,7 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         for (int j = 0; j < NT; ++j)
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
-                br[j][kk] = *(const bf16x8*)(bptr[j] + (size_t)(s * 2 + kk) * 512);
+                br[j][kk] = *(const bf16x8*)(bptr[j] + (size_t)(s * 2 + kk) * bstep);
     };
     const int lane_off[2] = {(r + 16 * g) * 8, ((r ^ 8) + 16 * g) * 8};
     auto compute = [&](int buf, bf16x8 (&br)[NT][2]) __attribute__((always_inline)) {
@@ -251,7 +255,7 @@ int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {256, 208, 128, 12
 int gemm_tile_bn(int tile) { static const int v[TILE_COUNT] = {256, 256, 256, 128, 256}; return v[tile]; }
 
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {
-    if (p.M <= 0 || p.N16 <= 0 || p.K32p <= 0 || (p.K32p & 1) || p.a_rows <= 0) return 1;
+    if (p.M <= 0 || p.N16 <= 0 || p.K32p <= 0 || (p.K32p & 1) || p.a_rows <= 0 || p.bgroup < 1) return 1;
     if (epi != EPI_PARTIAL && p.nsplit > 1) return 1;
     switch (epi) {
         case EPI_BIAS:      return launch_epi<EPI_BIAS>(p, tile, s);

@@ -15,9 +15,11 @@
 // multiple of 128 (the GEMM consumes 64-wide K stages in pairs) and N to a multiple of 16 with zeros.
 static inline int k32_padded(int K) { return ((K + 127) / 128) * 4; }
 static inline int n16_tiles(int N) { return (N + 15) / 16; }
-static inline size_t tiled_elems(int K, int N) { return (size_t)n16_tiles(N) * k32_padded(K) * 512; }
+// Tiles may further be grouped: with group size G the order is [nb / G][kb][nb % G], so that the G
+// column tiles one GEMM workgroup consumes per K step are contiguous in memory (N padded to 16 G).
+static inline size_t tiled_elems(int K, int N, int G = 1) { return (size_t)((n16_tiles(N) + G - 1) / G) * G * k32_padded(K) * 512; }
 
-void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, hipStream_t s);
+void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, hipStream_t s);
 
 // ----- large-M MFMA GEMM --------------------------------------------------------------
 enum GemmEpilogue {
@@ -33,6 +35,7 @@ enum GemmEpilogue {
 struct GemmP {
     const bf16_t* A; int lda; int a_rows;      // activations, rows clamped to a_rows - 1
     const bf16_t* B0; const bf16_t* B1;        // pre-tiled weights
+    int bgroup;                                // their tile group size G
     int M, N16, K32p;                          // valid rows, column tiles, padded k32 count
     int nsplit;                                // split-K factor (EPI_PARTIAL only when > 1)
     bf16_t* out; int ldo;

@@ -76,8 +76,10 @@ struct rtvla_ctx {
         bindex[name] = (int)bufs.size();
         bufs.push_back(b);
     }
-    void add_tiled(const char* name, int K, int N, int layers) {
-        add_buf(name, layers, (int64_t)tiled_elems(K, N), (int64_t)tiled_elems(K, N));
+    std::map<std::string, int> tgroup;          // tile group size of each re-tiled weight
+    void add_tiled(const char* name, int K, int N, int layers, int G = 1) {
+        add_buf(name, layers, (int64_t)tiled_elems(K, N, G), (int64_t)tiled_elems(K, N, G));
+        tgroup[name] = G;
     }
     bf16_t* TW(const char* n, int layer = 0) { const WsBuf& b = BI(n); return (bf16_t*)(ws + b.offset) + (size_t)b.ld * layer; }
 
@@ -208,17 +210,17 @@ int build_tables(rtvla_ctx* c) {
     if (pi05) c->add_tensor("valid_encoder_len", false, 4, {1});
 
     // ---- workspace: re-tiled weights first, then activations ----
-    c->add_tiled("t_vision_patch_embedding_w", 588, 1152, 1);
-    c->add_tiled("t_vision_attn_qkv_w", 1152, 3456, V);
-    c->add_tiled("t_vision_attn_o_w", 1152, 1152, V);
-    c->add_tiled("t_vision_ffn_up_w", 1152, 4304, V);
-    c->add_tiled("t_vision_ffn_down_w", 4304, 1152, V);
-    c->add_tiled("t_encoder_multi_modal_projector_w", 1152, 2048, 1);
-    c->add_tiled("t_encoder_attn_qkv_w", 2048, 2560, L);
-    c->add_tiled("t_encoder_attn_o_w", 2048, 2048, L);
-    c->add_tiled("t_encoder_ffn_gate_w", 2048, 16384, L);
-    c->add_tiled("t_encoder_ffn_up_w", 2048, 16384, L);
-    c->add_tiled("t_encoder_ffn_down_w", 16384, 2048, L);
+    c->add_tiled("t_vision_patch_embedding_w", 588, 1152, 1, 16);
+    c->add_tiled("t_vision_attn_qkv_w", 1152, 3456, V, 16);
+    c->add_tiled("t_vision_attn_o_w", 1152, 1152, V, 16);
+    c->add_tiled("t_vision_ffn_up_w", 1152, 4304, V, 16);
+    c->add_tiled("t_vision_ffn_down_w", 4304, 1152, V, 16);
+    c->add_tiled("t_encoder_multi_modal_projector_w", 1152, 2048, 1, 16);
+    c->add_tiled("t_encoder_attn_qkv_w", 2048, 2560, L, 16);
+    c->add_tiled("t_encoder_attn_o_w", 2048, 2048, L, 16);
+    c->add_tiled("t_encoder_ffn_gate_w", 2048, 16384, L, 8);
+    c->add_tiled("t_encoder_ffn_up_w", 2048, 16384, L, 8);
+    c->add_tiled("t_encoder_ffn_down_w", 16384, 2048, L, 16);
     c->add_tiled("t_decoder_attn_qkv_w", 1024, 2560, L);
     c->add_tiled("t_decoder_attn_o_w", 2048, 1024, L);
     c->add_tiled("t_decoder_ffn_gate_w", 1024, 4096, L);
@@ -280,9 +282,10 @@ struct Sched {
     Sched(rtvla_ctx* c_, hipStream_t s_) : c(c_), s(s_), d(c_->d), pi05(c_->d.model == RTVLA_PI05) {}
 
     void gemm(const bf16_t* A, int lda, int a_rows, int M, const bf16_t* B0, const bf16_t* B1, int K, int N, int epi, GemmP extra, const char* what) {
+        const int bgroup = epi == EPI_GEGLU ? 8 : 16;
         GemmP p = extra;
         p.A = A; p.lda = lda; p.a_rows = a_rows; p.M = M; p.B0 = B0; p.B1 = B1;
-        p.N16 = n16_tiles(N); p.K32p = k32_padded(K);
+        p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.bgroup = bgroup;
         const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU, epi == EPI_PARTIAL);
         p.nsplit = tc.nsplit;
         if (epi == EPI_PARTIAL) {
@@ -470,7 +473,7 @@ struct Sched {
         const int V = d.vision_layers, L = d.llm_layers;
         launch_fill_zero(c->ws + c->act_begin, c->ws_bytes - c->act_begin, s);
         auto tile = [&](const char* src, const char* dst, int K, int N, int layers) {
-            for (int i = 0; i < layers; ++i) launch_pretile(c->W(src, (size_t)K * N, i), K, N, c->TW(dst, i), s);
+            for (int i = 0; i < layers; ++i) launch_pretile(c->W(src, (size_t)K * N, i), K, N, c->TW(dst, i), c->tgroup.at(dst), s);
         };
         tile("vision_patch_embedding_w", "t_vision_patch_embedding_w", 588, 1152, 1);
         tile("vision_attn_qkv_w", "t_vision_attn_qkv_w", 1152, 3456, V);
@@ -499,7 +502,7 @@ struct Sched {
         launch_scale_inplace(c->B("decoder_out_proj_w_scaled"), 1024 * 32, dt, s);
         launch_copy_bytes(c->W("decoder_action_out_proj_b"), c->B("decoder_out_proj_b_scaled"), 64, s);
         launch_scale_inplace(c->B("decoder_out_proj_b_scaled"), 32, dt, s);
-        launch_pretile(c->B("decoder_out_proj_w_scaled"), 1024, 32, c->TW("t_decoder_out_proj_w"), s);
+        launch_pretile(c->B("decoder_out_proj_w_scaled"), 1024, 32, c->TW("t_decoder_out_proj_w"), 1, s);
         tile("decoder_time_mlp_in_w", "t_decoder_time_mlp_in_w", 1024, 1024, 1);
         tile("decoder_time_mlp_out_w", "t_decoder_time_mlp_out_w", 1024, 1024, 1);
         tile("decoder_pre_attn_norm_mod_w", "t_decoder_pre_attn_norm_mod_w", 1024, 3072, L);
@@ -757,7 +760,7 @@ size_t rtvla_pretile_elems(int K, int N) { return (K > 0 && N > 0) ? tiled_elems
 
 int rtvla_pretile(const void* w, int K, int N, void* w_tiled, void* stream) {
     if (!w || !w_tiled || K <= 0 || N <= 0) return RTVLA_ERR_ARG;
-    launch_pretile((const bf16_t*)w, K, N, (bf16_t*)w_tiled, (hipStream_t)stream);
+    launch_pretile((const bf16_t*)w, K, N, (bf16_t*)w_tiled, 1, (hipStream_t)stream);
     return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
 }
 

@@ -7,7 +7,7 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "librtvla.so")
+LIB_PATH = os.environ.get("RTVLA_LIBRARY") or os.path.join(HERE, "librtvla.so")   # override: an alternative build of the same ABI
 
 PI0, PI05 = 0, 1
 
