@@ -108,16 +108,22 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
             for (int i = 0; i < MT; ++i)
 #pragma unroll
                 for (int j = 0; j < NT; ++j) acc[i][j] = mfma16(br[j][kk], af[kk][i], acc[i][j]);
-        // instruction order for the scheduler: PRE fragment reads ahead, then NT MFMAs per further read
+        // instruction order for the scheduler: PRE fragment reads ahead, then per further read NT MFMAs
+        // and one of the next stage's global loads, so that load issue runs under the MFMAs
         constexpr int PRE = 4;
+        constexpr int NLOADS = AIT + 2 * NT;
         __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
         for (int t = 0; t < 2 * MT - PRE; ++t) {
             __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (t < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
 #pragma unroll
-        for (int t = 0; t < PRE; ++t) __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
+        for (int t = 0; t < PRE; ++t) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
+            if (t + 2 * MT - PRE < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
     };
 
     // K loop: the loads of stage s+1 fly under the MFMAs of stage s (register-staged A, weights in
@@ -133,13 +139,11 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         __syncthreads();
         for (int s = s_begin; s < s_end; s += 2) {          // the host guarantees an even stage count per split
             load_a(s + 1); load_b(s + 1, breg1);
-            __builtin_amdgcn_sched_barrier(0);
             compute(0, breg0);
             __builtin_amdgcn_sched_barrier(0);
             store_a(1);
             __syncthreads();
             load_a(min(s + 2, last)); load_b(min(s + 2, last), breg0);
-            __builtin_amdgcn_sched_barrier(0);
             compute(1, breg1);
             __builtin_amdgcn_sched_barrier(0);
             store_a(0);
