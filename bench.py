@@ -27,6 +27,7 @@ CONFIGS = {
 }
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+COPY_PROBE_BYTES = 256 << 20   # size of the calibration copy of --traffic-probe
 
 
 def main():
@@ -36,10 +37,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: launch the roofline kernel a few times, then a "
+                         "plain 256 MiB device copy whose counter reading calibrates the unit, and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one observation on ONE GPU; --gpus %d is not supported "
-              "(see DESIGN.md, 'More than one GPU')" % args.gpus, file=sys.stderr)
+              "(one observation is latency-bound work for a single device)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -63,6 +67,15 @@ def main():
         run = lambda nz: model.forward(img, nz)
     ctx = model._engine.ctx
     stream = torch.cuda.current_stream().cuda_stream
+    if args.traffic_probe:
+        ms, name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, 4, 5, stream)
+        src = torch.ones(COPY_PROBE_BYTES // 2, dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": name, "launch_ms": ms, "copy_bytes": COPY_PROBE_BYTES}))
+        return
     # fresh noise every iteration (BASELINE config 5); drawn up front so the timed region holds only forward()
     draws = [syn.observation(seed, views, chunk, device=dev, draw=i % 16)[2] for i in range(16)]
 
@@ -93,7 +106,11 @@ def main():
     mfma = geglu_flop / (geglu_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": "prefix GeGLU GEMM (gemm_mfma_kernel, EPI_GEGLU), M=%d K=2048 N=2x16384" % S_e,
                 "achieved": round(mfma, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(mfma / MFMA_PEAK_TFLOPS, 4),
-                "launch_ms": round(geglu_ms, 4), "traffic": None}
+                "launch_ms": round(geglu_ms, 4),
+                # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each calibrated on a 256 MiB copy; measured for
+                # the headline shape only (profiles/gemm_geglu_pi0_3view_p20_c50_hbm_traffic.md)
+                "traffic": 212.4e6 if args.config == "headline" else None,
+                "algorithmic_bytes": 2.0 * (S_e * 2048 + 2 * 2048 * 16384 + S_e * 16384)}
     # the action-expert side: one suffix layer (5 launches) streams 18 D_L-sized weight sets per step
     layer_ms = ctx.time_stage(capi.STAGE_SUFFIX_LAYER, 3, 0, 20, stream)
     d_l = 1024 * 2560 + 2048 * 1024 + 3 * 1024 * 4096
@@ -102,7 +119,7 @@ def main():
     roofline_hbm = {"bound": "hbm", "kernel": "one action-expert layer (qkv, attention, o, geglu, down)",
                     "achieved": round(hbm, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hbm / HBM_PEAK_GBS, 4),
                     "launch_ms": round(layer_ms, 4), "traffic": None}
-    # whole-forward roofline fraction (SURVEY 8d): (F_vis + F_pre) / P_mfma + B_dec / BW  over the measured p50
+    # whole-forward roofline fraction: (F_vis + F_pre) / P_mfma + B_dec / BW  over the measured p50
     v_l = 1152 * 3456 + 1152 * 1152 + 2 * 1152 * 4304
     e_l = 2048 * 2560 + 2048 * 2048 + 3 * 2048 * 16384
     f_vis = 2.0 * S_v * (588 * 1152 + 27 * v_l + 1152 * 2048) + 27 * views * 16 * 4 * 256 * 256 * 72
