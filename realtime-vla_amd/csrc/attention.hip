@@ -11,11 +11,35 @@
 // the softmax statistics are per-lane scalars and the probabilities are already in the register
 // layout of the MFMA B operand for O^T = V^T P^T, provided V is read with the matching key
 // permutation.  V is therefore kept transposed in memory ([d][key]) by the producing GEMM.
+//
+// The suffix pass has only ~26 row tiles but ~840 keys, and one CU can pull only ~100 GB/s through its
+// L2 port, so a workgroup that walks all keys is bound by that port.  Its keys are therefore split over
+// gridDim.y workgroups: each writes an un-normalised partial (O, row max, row sum) and takes a ticket
+// from a per-row-tile counter; the workgroup that draws the last ticket merges the partials and resets
+// the counter.  Nobody waits on anybody, so the grid always drains.  The partial records cross XCDs (each
+// has its own L2), so they are written and read with device-scope atomic accesses, which go through to the
+// memory-side coherence point: a device-scope release fence instead would write back the whole L2 once per
+// wave, which costs more than the attention itself.
 #include "kernels.h"
 
 namespace {
 
 constexpr float NEG_BIG = -1.0e30f;
+
+// device-coherent accesses to the key-split partial records
+RTVLA_DEVICE void coherent_store4(float* dst, f32x4 v) {
+    unsigned long long lo = ((unsigned long long)__float_as_uint(v[1]) << 32) | __float_as_uint(v[0]);
+    unsigned long long hi = ((unsigned long long)__float_as_uint(v[3]) << 32) | __float_as_uint(v[2]);
+    __hip_atomic_store((unsigned long long*)dst, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store((unsigned long long*)dst + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+RTVLA_DEVICE f32x4 coherent_load4(const float* src) {
+    const unsigned long long lo = __hip_atomic_load((const unsigned long long*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long hi = __hip_atomic_load((const unsigned long long*)src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return f32x4{__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)), __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
+}
+RTVLA_DEVICE void coherent_store(float* dst, float v) { __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+RTVLA_DEVICE float coherent_load(const float* src) { return __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 RTVLA_DEVICE bf16x8 cat44(bf16x4 lo, bf16x4 hi) {
     bf16x8 v;
@@ -35,6 +59,7 @@ void mqa_kernel(AttnP p) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
     const int m0 = blockIdx.x * (16 * MQ);
+    const int nsplit = gridDim.y, split = blockIdx.y;
 
     int vl = p.prefix_alloc;
     if (p.valid_len) vl = max(0, min(*p.valid_len, p.prefix_alloc));
@@ -58,6 +83,7 @@ void mqa_kernel(AttnP p) {
 
     constexpr int KBS = NTK * 16;                    // keys per block
     const int nkb = (p.keys + KBS - 1) / KBS;
+    const int kb_begin = split * p.kb_per_split, kb_end = min(nkb, kb_begin + p.kb_per_split);
     const int keys32 = p.ldvt >> 5;
     bf16x8 kf[NTK][8];        // K fragments of one key block (A operand of S^T = K Q^T)
     bf16x8 vf[16][NTK / 2];      // V^T fragments of the block, in the key order the P registers have
@@ -77,12 +103,12 @@ void mqa_kernel(AttnP p) {
             for (int kk = 0; kk < NTK / 2; ++kk) vf[dt][kk] = *(const bf16x8*)(vp + kk * 512);
         }
     };
-    if (w < nkb) { load_k(w); load_v(w); }
+    if (kb_begin + w < kb_end) { load_k(kb_begin + w); load_v(kb_begin + w); }
     __builtin_amdgcn_sched_barrier(0);
 
-    for (int kb = w; kb < nkb; kb += WAVES) {
+    for (int kb = kb_begin + w; kb < kb_end; kb += WAVES) {
         const int key0 = kb * KBS;
-        const int kb_next = min(kb + WAVES, nkb - 1);       // the last round re-reads a block instead of branching
+        const int kb_next = min(kb + WAVES, kb_end - 1);    // the last round re-reads a block instead of branching
         f32x4 st[MQ][NTK];
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
@@ -156,6 +182,7 @@ void mqa_kernel(AttnP p) {
         for (int mq = 0; mq < MQ; ++mq) ms[(w * MQ + mq) * 16 + r] = mrun[mq];
     }
     __syncthreads();
+    float mgl[MQ];
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         float mg = NEG_BIG;
@@ -166,7 +193,11 @@ void mqa_kernel(AttnP p) {
 #pragma unroll
         for (int dt = 0; dt < 16; ++dt) o[mq][dt] *= sc;
         if (g == 0) ls[(w * MQ + mq) * 16 + r] = lrun[mq];
+        mgl[mq] = mg;
     }
+    // partial record of one (row block, split): MQ x { O [16][64] f32x4 | max [16] | sum [16] }
+    constexpr int REC = 16 * 64 * 4 + 32;
+    float* const mine = p.partial + ((size_t)blockIdx.x * nsplit + split) * (MQ * REC);
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         __syncthreads();                       // ls written / previous obuf round consumed
@@ -178,13 +209,63 @@ void mqa_kernel(AttnP p) {
         for (int ww = 0; ww < WAVES; ++ww) lt += ls[(ww * MQ + mq) * 16 + r];
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         const int row = m0 + mq * 16 + r;
+        if (nsplit > 1 && w == 0 && g == 0) {
+            if (p.dbg & 1) { mine[mq * REC + 4096 + r] = mgl[mq]; mine[mq * REC + 4112 + r] = lt; }
+            else { coherent_store(mine + mq * REC + 4096 + r, mgl[mq]); coherent_store(mine + mq * REC + 4112 + r, lt); }
+        }
         for (int dt = w; dt < 16; dt += WAVES) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ww = 0; ww < WAVES; ++ww) t += obuf[((size_t)ww * 16 + dt) * 64 + lane];
-            if (row < p.rows) {
+            if (nsplit > 1) {
+                if (p.dbg & 1) *(f32x4*)(mine + mq * REC + (dt * 64 + lane) * 4) = t;
+                else coherent_store4(mine + mq * REC + (dt * 64 + lane) * 4, t);
+            } else if (row < p.rows) {
                 const int d = dt * 16 + 4 * g;
                 // tiled output: the [tokens][8*256] matrix the suffix O-projection reads as MFMA fragments
+                bf16_t* dst = p.out_tiled ? p.out + ft_index(row >> 3, (row & 7) * 256 + d, 64) : p.out + (size_t)row * p.ldo + d;
+                store4(dst, pack4(t * inv));
+            }
+        }
+    }
+    if (nsplit == 1 || (p.dbg & 2)) return;
+
+    // ---- ticket: the last workgroup of this row block to finish merges all splits ----
+    __shared__ unsigned last_flag;
+    __builtin_amdgcn_s_waitcnt(0);             // every wave's partial stores have been acknowledged by the coherence point
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned old = __hip_atomic_fetch_add(p.counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned last = old == (unsigned)(nsplit - 1);
+        if (last) __hip_atomic_store(p.counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+        last_flag = last;
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const float* const all = p.partial + (size_t)blockIdx.x * nsplit * (MQ * REC);
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+        float mg = NEG_BIG;
+        for (int sp = 0; sp < nsplit; ++sp) mg = fmaxf(mg, coherent_load(all + (size_t)sp * (MQ * REC) + mq * REC + 4096 + r));
+        float lt = 0.f;
+        for (int sp = 0; sp < nsplit; ++sp) {
+            const float* rec = all + (size_t)sp * (MQ * REC) + mq * REC;
+            lt += __expf(coherent_load(rec + 4096 + r) - mg) * coherent_load(rec + 4112 + r);
+        }
+        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+        const int row = m0 + mq * 16 + r;
+        for (int dt = w; dt < 16; dt += WAVES) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+            for (int sp = 0; sp < nsplit; ++sp) {
+                const float* rec = all + (size_t)sp * (MQ * REC) + mq * REC;
+                if (p.dbg & 1) t += *(const f32x4*)(rec + (dt * 64 + lane) * 4) * __expf(coherent_load(rec + 4096 + r) - mg);
+                else t += coherent_load4(rec + (dt * 64 + lane) * 4) * __expf(coherent_load(rec + 4096 + r) - mg);
+            }
+            if (row < p.rows) {
+                const int d = dt * 16 + 4 * g;
                 bf16_t* dst = p.out_tiled ? p.out + ft_index(row >> 3, (row & 7) * 256 + d, 64) : p.out + (size_t)row * p.ldo + d;
                 store4(dst, pack4(t * inv));
             }
@@ -275,7 +356,7 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 }
 
 template <int WAVES, int MQ, int NTK>
-int launch_mqa_inst(const AttnP& p, hipStream_t s) {
+int launch_mqa_inst(AttnP p, hipStream_t s) {
     const size_t smem = (size_t)WAVES * 16 * 64 * 16 + (size_t)2 * WAVES * MQ * 16 * 4;
     auto kern = mqa_kernel<WAVES, MQ, NTK>;
     if (smem > 65536) {
@@ -283,7 +364,15 @@ int launch_mqa_inst(const AttnP& p, hipStream_t s) {
         if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
     }
     const int blocks = (p.rows + 16 * MQ - 1) / (16 * MQ);
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(WAVES * 64), smem, s, p);
+    const int nkb = (p.keys + NTK * 16 - 1) / (NTK * 16);
+    const int want = p.nsplit > 1 ? p.nsplit : 1;
+    p.kb_per_split = (nkb + want - 1) / want;
+    const int nsplit = (nkb + p.kb_per_split - 1) / p.kb_per_split;
+    if (nsplit > 1) {
+        if (!p.partial || !p.counters) return 1;
+        if ((size_t)blocks * nsplit * MQ * (16 * 64 * 4 + 32) > p.partial_floats || blocks > p.counter_count) return 3;
+    }
+    hipLaunchKernelGGL(kern, dim3(blocks, nsplit), dim3(WAVES * 64), smem, s, p);
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 
@@ -291,8 +380,13 @@ int launch_mqa_inst(const AttnP& p, hipStream_t s) {
 
 int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s) {
     if (p.rows <= 0 || p.keys <= 0 || (p.ldvt & 63) || p.ldvt < ((p.keys + 63) / 64) * 64) return 1;
-    if (waves == 8) return launch_mqa_inst<4, 1, 4>(p, s);      // suffix pass: few rows, one row tile per workgroup
-    if (waves == 4) return launch_mqa_inst<4, 2, 2>(p, s);
+    switch (waves) {                                            // variant: waves, row tiles and 16-key tiles per wave round
+        case 4: return launch_mqa_inst<4, 2, 2>(p, s);          // prefix pass
+        case 8: return launch_mqa_inst<4, 1, 4>(p, s);          // suffix pass: few rows, one row tile per workgroup
+        case 9: return launch_mqa_inst<2, 1, 4>(p, s);
+        case 10: return launch_mqa_inst<4, 1, 2>(p, s);
+        case 11: return launch_mqa_inst<2, 2, 2>(p, s);
+    }
     return 2;
 }
 

@@ -2,7 +2,10 @@
 // kernels of /root/reference/pi0_infer.py:82-124, :693-725, :939-1039, :1122-1163 and
 // /root/reference/pi05_infer.py:22-64, :78-113, :127-195.
 //
-// One workgroup owns one 16-column tile of the output and all of K; its 8 waves split K.  Each wave
+// One workgroup owns one 16-column tile of the output, MTS 16-row tiles and all of K; its 8 waves split K.
+// (A workgroup has to pull its rows of the activations through its own CU's L2 port, which moves only
+// ~100 GB/s: the few-column projections (O, down: 64 column tiles) therefore run one row tile per
+// workgroup so that 256 CUs share that traffic, the wide ones keep all rows and read the weights once.)  Each wave
 // issues all of its weight-fragment loads up front (coalesced 1 KB reads of the pre-tiled layout,
 // straight into registers), reads its slice of the activations in MFMA operand order from L2,
 // multiplies, and the waves reduce through LDS.  Because the workgroup sees every activation row
@@ -14,10 +17,9 @@
 namespace {
 
 constexpr int SK_WAVES = 8;
-constexpr int SK_MTS = 4;      // 4 x 16 = 64 rows
 constexpr int SK_CH = 4;       // k32 blocks per A-prefetch chunk
 
-template <int NCH, int NORM, int EPI>
+template <int NCH, int NORM, int EPI, int SK_MTS>
 __global__ __launch_bounds__(SK_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void skinny_kernel(SkinnyP p) {
     constexpr int KBW = NCH * SK_CH;
@@ -31,6 +33,7 @@ void skinny_kernel(SkinnyP p) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
     const int tile = blockIdx.x;
+    const int m_base = blockIdx.y * (SK_MTS * 16);
     const int kb0 = w * KBW;
 
     // ---- weight fragments: the HBM stream, all in flight at once ----
@@ -51,7 +54,7 @@ void skinny_kernel(SkinnyP p) {
     const int astep = p.a_tiled ? 512 : 32;
 #pragma unroll
     for (int mt = 0; mt < SK_MTS; ++mt) {
-        const int row = min(mt * 16 + r, p.M - 1) + p.a_row0;
+        const int row = min(m_base + mt * 16 + r, p.M - 1) + p.a_row0;
         arow[mt] = p.a_tiled ? p.A + ft_index(row, kb0 * 32 + 8 * g, p.lda >> 5) : p.A + (size_t)row * p.lda + kb0 * 32 + 8 * g;
     }
     f32x4 acc[NB][SK_MTS];
@@ -136,7 +139,7 @@ void skinny_kernel(SkinnyP p) {
     __syncthreads();
     if (w >= SK_MTS) return;
     const int mt = w;
-    const int m = mt * 16 + r;
+    const int m = m_base + mt * 16 + r;
     f32x4 v[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -183,16 +186,16 @@ void skinny_kernel(SkinnyP p) {
     }
 }
 
-template <int NCH, int NORM, int EPI>
+template <int NCH, int NORM, int EPI, int SK_MTS>
 int launch_inst(const SkinnyP& p, hipStream_t s) {
     constexpr int NB = (EPI == SK_GEGLU) ? 2 : 1;
     const size_t smem = (size_t)SK_WAVES * NB * SK_MTS * 64 * 16 + (size_t)SK_WAVES * 64 * 4;
-    auto kern = skinny_kernel<NCH, NORM, EPI>;
+    auto kern = skinny_kernel<NCH, NORM, EPI, SK_MTS>;
     if (smem > 65536) {
         static bool done = false;
         if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
     }
-    hipLaunchKernelGGL(kern, dim3(p.N16), dim3(SK_WAVES * 64), smem, s, p);
+    hipLaunchKernelGGL(kern, dim3(p.N16, (p.M + SK_MTS * 16 - 1) / (SK_MTS * 16)), dim3(SK_WAVES * 64), smem, s, p);
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 
@@ -206,17 +209,17 @@ int launch_skinny(const SkinnyP& p, int epi, hipStream_t s) {
     const int nch = p.K / (32 * SK_WAVES * SK_CH);
     if (p.norm != SN_NONE && nch != 1) return 1;
     if (p.norm == SN_ADARMS && !p.style) return 1;
-#define SK_CASE(NCH_, NORM_, EPI_) if (nch == NCH_ && p.norm == NORM_ && epi == EPI_) return launch_inst<NCH_, NORM_, EPI_>(p, s)
-    SK_CASE(1, SN_RMS, SK_QKV_ROPE);
-    SK_CASE(1, SN_ADARMS, SK_QKV_ROPE);
-    SK_CASE(1, SN_RMS, SK_GEGLU);
-    SK_CASE(1, SN_ADARMS, SK_GEGLU);
-    SK_CASE(1, SN_NONE, SK_BIAS);
-    SK_CASE(1, SN_NONE, SK_BIAS_SILU);
-    SK_CASE(1, SN_RMS, SK_RES);
-    SK_CASE(1, SN_ADARMS, SK_RES);
-    SK_CASE(2, SN_NONE, SK_RES);
-    SK_CASE(4, SN_NONE, SK_RES);
+#define SK_CASE(NCH_, NORM_, EPI_, MTS_) if (nch == NCH_ && p.norm == NORM_ && epi == EPI_) return launch_inst<NCH_, NORM_, EPI_, MTS_>(p, s)
+    SK_CASE(1, SN_RMS, SK_QKV_ROPE, 4);
+    SK_CASE(1, SN_ADARMS, SK_QKV_ROPE, 4);
+    SK_CASE(1, SN_RMS, SK_GEGLU, 4);
+    SK_CASE(1, SN_ADARMS, SK_GEGLU, 4);
+    SK_CASE(1, SN_NONE, SK_BIAS, 4);
+    SK_CASE(1, SN_NONE, SK_BIAS_SILU, 4);
+    SK_CASE(1, SN_RMS, SK_RES, 4);
+    SK_CASE(1, SN_ADARMS, SK_RES, 4);
+    SK_CASE(2, SN_NONE, SK_RES, 1);
+    SK_CASE(4, SN_NONE, SK_RES, 1);
 #undef SK_CASE
     return 2;
 }
