@@ -1,26 +1,30 @@
 // Large-M bf16 GEMM on MFMA for the SigLIP and Gemma-prefix layers
 // (replaces the Triton GEMM family of /root/reference/pi0_infer.py:5-346, :664-691, :777-810).
 //
-// out[M][N] = epilogue(A[M][K] * W[K][N]).  The activations A are staged through LDS in MFMA
-// operand-fragment order (each wave reads whole 1 KB fragments with ds_read_b128, conflict
-// free) and are shared by all waves of the workgroup; the weights are read straight from
-// their pre-tiled layout in HBM into registers (one coalesced 1 KB load per fragment, no LDS
-// round trip), each wave owning its own column tiles.  The product is computed transposed
-// (weights as the MFMA A operand) so that every lane ends up with 4 consecutive output columns
-// of one row: 8-byte packed stores, and RoPE pairs / GeGLU partners sit in the same lane.
+// out[M][N] = epilogue(A[M][K] * W[K][N]) with v_mfma_f32_32x32x16_bf16: measured on MI355X this
+// instruction sustains ~2.1 PFLOP/s with a single wave per SIMD, while streams of independent
+// 16x16x32 MFMAs issue at half that rate.  The activations A are staged through LDS in MFMA
+// operand-fragment order (each wave reads whole 1 KB fragments with ds_read_b128, conflict free) and
+// are shared by all waves of the workgroup; the weights are read straight from their pre-tiled layout
+// in HBM into registers (one coalesced 1 KB load per fragment, no LDS round trip), each wave owning
+// its own column tiles.  The product is computed transposed (weights as the MFMA A operand) so that
+// every lane ends up with 4 groups of 4 consecutive output columns of one row: 8-byte packed stores,
+// and RoPE pairs / GeGLU partners sit in the same lane.
 #include "kernels.h"
 
 namespace {
 
 template <int EPI> struct EpiTraits { static constexpr bool dual = (EPI == EPI_GEGLU); };
 
-// tiles of at most 128 rows are compiled to fit two workgroups per CU (<= 256 registers per lane) so
-// that one workgroup's MFMAs run under the other's memory latency
+RTVLA_DEVICE f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+
+// MT, NT: 32-row tiles per workgroup and 32-column tiles per wave.  Small tiles are compiled to fit two
+// workgroups per CU so that one workgroup's MFMAs run under the other's memory latency.
 template <int WN, int MT, int NT, int EPI>
-__global__ __launch_bounds__(WN * 64, (MT <= 8 ? 2 : 1))
+__global__ __launch_bounds__(WN * 64, (MT <= 2 && WN == 4 ? 2 : 1))
 void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int stages_per_split) {
     constexpr int NTH = WN * 64;
-    constexpr int BM = MT * 16;
+    constexpr int BM = MT * 32;
     constexpr int A_CHUNKS = BM * 8;                       // 16-byte chunks per 64-wide K stage
     constexpr int AIT = (A_CHUNKS + NTH - 1) / NTH;
     constexpr int STAGE_ELEMS = BM * 64;
@@ -28,7 +32,7 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
     bf16_t* lds = (bf16_t*)smem_raw;
 
     const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
-    const int g = lane >> 4, r = lane & 15;
+    const int h = lane >> 5, r = lane & 31;
 
     const int total = m_blocks * n_blocks * p.nsplit;
     const int lid = xcd_remap(blockIdx.x, total);
@@ -40,132 +44,144 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
     const int s_begin = split * stages_per_split;
     const int s_end = min(s_begin + stages_per_split, stages_total);
 
-    // column tiles of this wave
+    // 32-column tiles of this wave
     constexpr int HALF = EpiTraits<EPI>::dual ? NT / 2 : NT;
     int tile_of[NT];
     const bf16_t* bptr[NT];
+    const int n32 = (p.N16 + 1) >> 1;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         const int t = (n_blk * WN + wn) * HALF + (j % HALF);
         tile_of[j] = t;
         const bf16_t* base = (EpiTraits<EPI>::dual && j >= HALF) ? p.B1 : p.B0;
         const int G = p.bgroup;
-        const int tc = min(t, ((p.N16 + G - 1) / G) * G - 1);
-        bptr[j] = base + ((size_t)(tc / G) * p.K32p * G + (tc % G)) * 512 + lane * 8;
+        const int tc = min(t, ((n32 + G - 1) / G) * G - 1);
+        bptr[j] = base + ((size_t)(tc / G) * (p.K32p * 2) * G + (tc % G)) * 512 + lane * 8;
     }
 
-    const size_t bstep = (size_t)p.bgroup * 512;          // distance between consecutive k32 blocks of one column tile
-    f32x4 acc[MT][NT];
+    const size_t bstep = (size_t)p.bgroup * 512;          // distance between consecutive k16 blocks of one column tile
+    f32x16 acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < NT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    bf16x8 areg[AIT];
-    bf16x8 breg0[NT][2], breg1[NT][2];
+    bf16x8 areg0[AIT], areg1[AIT];
+    bf16x8 breg0[NT][4], breg1[NT][4];
 
-    // LDS stage layout: fragment (row tile i, k half kk) is 1 KB, lane (g, r) at slot (r ^ 8 kk) + 16 g.
-    // The xor spreads the 64 lanes of a staging write (8 rows x 8 chunks) over all banks; a
-    // fragment read still touches every bank exactly once.
-    auto load_a = [&](int s) __attribute__((always_inline)) {
+    // LDS stage layout: fragment (row tile i, k16 step ks) is 1 KB = 64 slots of 16 bytes; the chunk of row r
+    // (0..31) and k half hh sits at slot 8 ((r >> 3) + 4 hh) + ((r + 2 ks + hh) & 7).  The low three bits pick
+    // the 128-byte bank group: any 8 consecutive lanes of a fragment read (8 rows, one hh) and any 8
+    // consecutive lanes of a staging write (one row, 8 chunks = 4 ks x 2 hh) land in 8 different bank
+    // groups, so neither side conflicts.
+    auto load_a = [&](int s, bf16x8 (&ar)[AIT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < AIT; ++it) {
             // a ragged last round re-reads the final chunk instead of branching
             const int c = min(it * NTH + tid, A_CHUNKS - 1);
             const int row = c >> 3, kc = c & 7;
             const int gr = min(m0 + row, p.a_rows - 1);
-            areg[it] = *(const bf16x8*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
+            ar[it] = *(const bf16x8*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
         }
     };
-    auto store_a = [&](int buf) __attribute__((always_inline)) {
+    auto store_a = [&](int buf, bf16x8 (&ar)[AIT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < AIT; ++it) {
             const int c = min(it * NTH + tid, A_CHUNKS - 1);      // duplicates write identical data
-            const int row = c >> 3, kc = c & 7, kk = kc >> 2;
-            const int off = ((((row >> 4) * 2 + kk) * 64) + ((row & 15) ^ (kk << 3)) + 16 * (kc & 3)) * 8;
-            *(bf16x8*)(lds + buf * STAGE_ELEMS + off) = areg[it];
+            const int row = c >> 3, kc = c & 7, ks = kc >> 1, hh = kc & 1;
+            const int rr = row & 31;
+            const int off = ((((row >> 5) * 4 + ks) * 64) + 8 * ((rr >> 3) + 4 * hh) + ((rr + 2 * ks + hh) & 7)) * 8;
+            *(bf16x8*)(lds + buf * STAGE_ELEMS + off) = ar[it];
         }
     };
-    auto load_b = [&](int s, bf16x8 (&br)[NT][2]) __attribute__((always_inline)) {
+    auto load_b_half = [&](int s, bf16x8 (&br)[NT][4], int kk) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < NT; ++j)
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
-                br[j][kk] = *(const bf16x8*)(bptr[j] + (size_t)(s * 2 + kk) * bstep);
+            for (int q = 0; q < 2; ++q) br[j][2 * kk + q] = *(const bf16x8*)(bptr[j] + (size_t)(s * 4 + 2 * kk + q) * bstep);
     };
-    const int lane_off[2] = {(r + 16 * g) * 8, ((r ^ 8) + 16 * g) * 8};
-    auto compute = [&](int buf, bf16x8 (&br)[NT][2]) __attribute__((always_inline)) {
+    int lane_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) lane_off[ks] = (8 * ((r >> 3) + 4 * h) + ((r + 2 * ks + h) & 7)) * 8;
+    // One K stage.  Both operands are prefetched TWO stages ahead: the activations of stage t+2 go to the
+    // register set whose contents (stage t) already sit in LDS, and each half of the weight registers is
+    // re-loaded with stage t+2 as soon as the MFMAs of stage t have consumed it, so no third register set
+    // is needed.  The scheduler is given the instruction order explicitly: fragment reads run PRE ahead of
+    // the MFMAs that use them and the global loads are spread one per MFMA group.
+    auto stage = [&](int buf, int s_next, bf16x8 (&br)[NT][4], bf16x8 (&ar_next)[AIT], bf16x8 (&ar_store)[AIT]) __attribute__((always_inline)) {
         const bf16_t* base = lds + buf * STAGE_ELEMS;
-        // all A fragments of the stage are requested from LDS before the first MFMA waits on one
-        bf16x8 af[2][MT];
+        load_a(s_next, ar_next);
+        bf16x8 af[4][MT];
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int i = 0; i < MT; ++i) af[kk][i] = *(const bf16x8*)(base + (i * 2 + kk) * 512 + lane_off[kk]);
+            for (int i = 0; i < MT; ++i) af[ks][i] = *(const bf16x8*)(base + (i * 4 + ks) * 512 + lane_off[ks]);
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
+        for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
             for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int j = 0; j < NT; ++j) acc[i][j] = mfma16(br[j][kk], af[kk][i], acc[i][j]);
-        // instruction order for the scheduler: PRE fragment reads ahead, then per further read NT MFMAs
-        // and one of the next stage's global loads, so that load issue runs under the MFMAs
-        constexpr int PRE = 4;
-        constexpr int NLOADS = AIT + 2 * NT;
+                for (int j = 0; j < NT; ++j) acc[i][j] = mfma32(br[j][ks], af[ks][i], acc[i][j]);
+        load_b_half(s_next, br, 0);
+#pragma unroll
+        for (int ks = 2; ks < 4; ++ks)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[i][j] = mfma32(br[j][ks], af[ks][i], acc[i][j]);
+        load_b_half(s_next, br, 1);
+        constexpr int PRE = 3;
+        constexpr int R = 4 * MT;                                       // fragment reads of the stage
+        static_assert(R / 2 >= 2 * NT && AIT <= R / 2, "not enough MFMA groups to spread the loads over");
         __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
-        for (int t = 0; t < 2 * MT - PRE; ++t) {
+        for (int t = 0; t < R; ++t) {
             __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (t < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (t < R - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (t < AIT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                        // activation loads
+            if (t >= R / 2 && t < R / 2 + 2 * NT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // weight loads, k half 0
         }
-#pragma unroll
-        for (int t = 0; t < PRE; ++t) {
-            __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
-            if (t + 2 * MT - PRE < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
+        __builtin_amdgcn_sched_group_barrier(0x020, 2 * NT, 0);                                    // weight loads, k half 1
+        __builtin_amdgcn_sched_barrier(0);
+        store_a(buf ^ 1, ar_store);
+        __syncthreads();
     };
 
-    // K loop: the loads of stage s+1 fly under the MFMAs of stage s (register-staged A, weights in
-    // a second register set); two stages per trip so the sets alternate without a runtime index and
-    // the body has a single exit.  Past the end the prefetch re-reads the last stage instead of
-    // branching around the loads.
+    // K loop, two stages per trip so the register sets and LDS buffers alternate without a runtime index and
+    // the body has a single exit.  Past the end the prefetch re-reads the last stage instead of branching.
     const int n_st = s_end - s_begin;
     if (n_st > 0) {
         const int last = s_end - 1;
-        load_a(s_begin);
-        load_b(s_begin, breg0);
-        store_a(0);
+        load_a(s_begin, areg0);
+        load_b_half(s_begin, breg0, 0); load_b_half(s_begin, breg0, 1);
+        load_a(min(s_begin + 1, last), areg1);
+        load_b_half(min(s_begin + 1, last), breg1, 0); load_b_half(min(s_begin + 1, last), breg1, 1);
+        store_a(0, areg0);
         __syncthreads();
         for (int s = s_begin; s < s_end; s += 2) {          // the host guarantees an even stage count per split
-            load_a(s + 1); load_b(s + 1, breg1);
-            compute(0, breg0);
-            __builtin_amdgcn_sched_barrier(0);
-            store_a(1);
-            __syncthreads();
-            load_a(min(s + 2, last)); load_b(min(s + 2, last), breg0);
-            compute(1, breg1);
-            __builtin_amdgcn_sched_barrier(0);
-            store_a(0);
-            __syncthreads();
+            stage(0, min(s + 2, last), breg0, areg0, areg1);
+            stage(1, min(s + 3, last), breg1, areg1, areg0);
         }
     }
 
-    // ---- epilogue: lane (g, r) holds rows m = m0 + 16 i + r, columns n = 16 tile + 4 g + v ----
+    // ---- epilogue: lane (h, r) holds rows m = m0 + 32 i + r, columns n = 32 tile + 8 grp + 4 h + e ----
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        const int m = m0 + i * 16 + r;
+        const int m = m0 + i * 32 + r;
         if (m >= p.M) continue;
 #pragma unroll
         for (int j = 0; j < HALF; ++j) {
-            const int t = tile_of[j];
-            if (t >= p.N16) continue;
-            const int n0 = t * 16 + 4 * g;
-            f32x4 v = acc[i][j];
+#pragma unroll
+          for (int grp = 0; grp < 4; ++grp) {
+            const int n0 = tile_of[j] * 32 + 8 * grp + 4 * h;
+            if (n0 >= p.N16 * 16) continue;
+            f32x4 v = {acc[i][j][4 * grp], acc[i][j][4 * grp + 1], acc[i][j][4 * grp + 2], acc[i][j][4 * grp + 3]};
             if constexpr (EPI == EPI_PARTIAL) {
                 *(f32x4*)(p.partial + (size_t)split * p.pstride + (size_t)m * p.ldp + n0) = v;
             } else if constexpr (EPI == EPI_GEGLU) {
-                const f32x4 u = acc[i][j + HALF];
+                const f32x4 u = {acc[i][j + HALF][4 * grp], acc[i][j + HALF][4 * grp + 1], acc[i][j + HALF][4 * grp + 2], acc[i][j + HALF][4 * grp + 3]};
                 store4(p.out + (size_t)m * p.ldo + n0,
                        pack4(gelu_tanh(v[0]) * u[0], gelu_tanh(v[1]) * u[1], gelu_tanh(v[2]) * u[2], gelu_tanh(v[3]) * u[3]));
             } else if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_PATCH) {
@@ -215,16 +231,17 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
                     for (int e = 0; e < 4; ++e) p.vt[vh * (80 * 256) + vt_index(d + e, tok, 8)] = f2bf(v[e]);
                 }
             }
+          }
         }
     }
 }
 
 template <int WN, int MT, int NT, int EPI>
 int launch_cfg(const GemmP& p, hipStream_t s) {
-    constexpr int BM = MT * 16;
+    constexpr int BM = MT * 32;
     constexpr int HALF = EpiTraits<EPI>::dual ? NT / 2 : NT;
     const int m_blocks = (p.M + BM - 1) / BM;
-    const int n_blocks = (p.N16 + WN * HALF - 1) / (WN * HALF);
+    const int n_blocks = ((p.N16 + 1) / 2 + WN * HALF - 1) / (WN * HALF);
     const int stages_total = p.K32p / 2;
     const int nsplit = p.nsplit < 1 ? 1 : p.nsplit;
     const int sps = (stages_total + nsplit - 1) / nsplit;
@@ -244,19 +261,20 @@ int launch_cfg(const GemmP& p, hipStream_t s) {
 template <int EPI>
 int launch_epi(const GemmP& p, int tile, hipStream_t s) {
     switch (tile) {
-        case TILE_256x256: return launch_cfg<4, 16, 4, EPI>(p, s);
-        case TILE_208x256: return launch_cfg<4, 13, 4, EPI>(p, s);
-        case TILE_128x256: return launch_cfg<4, 8, 4, EPI>(p, s);
-        case TILE_128x128: return launch_cfg<4, 8, 2, EPI>(p, s);
-        case TILE_64x256:  return launch_cfg<4, 4, 4, EPI>(p, s);
+        case TILE_256x256: return launch_cfg<4, 8, 2, EPI>(p, s);
+        case TILE_224x256: return launch_cfg<4, 7, 2, EPI>(p, s);
+        case TILE_160x256: return launch_cfg<4, 5, 2, EPI>(p, s);
+        case TILE_128x256: return launch_cfg<4, 4, 2, EPI>(p, s);
+        case TILE_96x256:  return launch_cfg<4, 3, 2, EPI>(p, s);
+        case TILE_64x256:  return launch_cfg<4, 2, 2, EPI>(p, s);
     }
     return 2;
 }
 
 }  // namespace
 
-int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {256, 208, 128, 128, 64}; return v[tile]; }
-int gemm_tile_bn(int tile) { static const int v[TILE_COUNT] = {256, 256, 256, 128, 256}; return v[tile]; }
+int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {256, 224, 160, 128, 96, 64}; return v[tile]; }
+int gemm_tile_bn(int tile) { return 256; }
 
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {
     if (p.M <= 0 || p.N16 <= 0 || p.K32p <= 0 || (p.K32p & 1) || p.a_rows <= 0 || p.bgroup < 1) return 1;

@@ -18,8 +18,11 @@ static inline int n16_tiles(int N) { return (N + 15) / 16; }
 // Tiles may further be grouped: with group size G the order is [nb / G][kb][nb % G], so that the G
 // column tiles one GEMM workgroup consumes per K step are contiguous in memory (N padded to 16 G).
 static inline size_t tiled_elems(int K, int N, int G = 1) { return (size_t)((n16_tiles(N) + G - 1) / G) * G * k32_padded(K) * 512; }
+// The large-M GEMM uses 32x32x16 MFMAs and therefore "wide" tiles: 32 columns x 16 rows, lane l carrying
+// W[kb*16 + 8 (l >> 5) + j][nb*32 + (l & 31)], stored [nb / G][kb][nb % G] with the same K padding.
+static inline size_t tiled_elems_wide(int K, int N, int G) { return (size_t)(((N + 31) / 32 + G - 1) / G) * G * k32_padded(K) * 2 * 512; }
 
-void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, hipStream_t s);
+void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide, hipStream_t s);
 
 // ----- large-M MFMA GEMM --------------------------------------------------------------
 enum GemmEpilogue {
@@ -35,7 +38,7 @@ enum GemmEpilogue {
 struct GemmP {
     const bf16_t* A; int lda; int a_rows;      // activations, rows clamped to a_rows - 1
     const bf16_t* B0; const bf16_t* B1;        // pre-tiled weights
-    int bgroup;                                // their tile group size G
+    int bgroup;                                // their (wide) tile group size G
     int M, N16, K32p;                          // valid rows, column tiles, padded k32 count
     int nsplit;                                // split-K factor (EPI_PARTIAL only when > 1)
     bf16_t* out; int ldo;
@@ -45,8 +48,8 @@ struct GemmP {
     const bf16_t* rope;                        // [row][256] = cos0 sin0 cos1 sin1 ...
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt;
 };
-// tile configuration: 0 = 256x256 block (4 waves x 16x4 tiles), 1 = 208x256, 2 = 128x256, 3 = 128x128 (2x2 waves? no: 4 waves x 8x2)
-enum GemmTile { TILE_256x256 = 0, TILE_208x256, TILE_128x256, TILE_128x128, TILE_64x256, TILE_COUNT };
+// workgroup tile (rows x columns), 4 waves each owning 64 columns (two 32-column MFMA tiles)
+enum GemmTile { TILE_256x256 = 0, TILE_224x256, TILE_160x256, TILE_128x256, TILE_96x256, TILE_64x256, TILE_COUNT };
 int gemm_tile_bm(int tile);
 int gemm_tile_bn(int tile);
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s);

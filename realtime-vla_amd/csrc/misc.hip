@@ -6,16 +6,16 @@ namespace {
 
 // ---------------------------------------------------------------------------------------------
 // W[K][N] -> MFMA fragment tiles [nb][kb][lane][8] (see kernels.h)
-__global__ void pretile_kernel(const bf16_t* __restrict__ W, int K, int N, bf16_t* __restrict__ out, int K32p, int G, size_t chunks) {
+__global__ void pretile_kernel(const bf16_t* __restrict__ W, int K, int N, bf16_t* __restrict__ out, int KBp, int G, int wide, size_t chunks) {
     const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= chunks) return;
     const int lane = (int)(c & 63);
     const size_t tile = c >> 6;                             // order [nb / G][kb][nb % G]
-    const size_t per_group = (size_t)K32p * G;
+    const size_t per_group = (size_t)KBp * G;              // KBp: padded K in blocks of 32 (or of 16 for wide tiles)
     const int group = (int)(tile / per_group), rem = (int)(tile % per_group);
     const int kb = rem / G, nb = group * G + rem % G;
-    const int n = nb * 16 + (lane & 15);
-    const int k0 = kb * 32 + 8 * (lane >> 4);
+    const int n = wide ? nb * 32 + (lane & 31) : nb * 16 + (lane & 15);
+    const int k0 = wide ? kb * 16 + 8 * (lane >> 5) : kb * 32 + 8 * (lane >> 4);
     bf16x8 v;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -166,10 +166,10 @@ __global__ void scale_kernel(bf16_t* p, size_t n, float f) {
 
 }  // namespace
 
-void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, hipStream_t s) {
-    const int K32p = k32_padded(K);
-    const size_t chunks = tiled_elems(K, N, G) / 8;
-    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, K32p, G, chunks);
+void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide, hipStream_t s) {
+    const int KBp = wide ? k32_padded(K) * 2 : k32_padded(K);
+    const size_t chunks = (wide ? tiled_elems_wide(K, N, G) : tiled_elems(K, N, G)) / 8;
+    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, KBp, G, wide, chunks);
 }
 
 int launch_reduce(const ReduceP& p, hipStream_t s) {

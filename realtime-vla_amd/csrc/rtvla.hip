@@ -77,9 +77,11 @@ struct rtvla_ctx {
         bufs.push_back(b);
     }
     std::map<std::string, int> tgroup;          // tile group size of each re-tiled weight
-    void add_tiled(const char* name, int K, int N, int layers, int G = 1) {
-        add_buf(name, layers, (int64_t)tiled_elems(K, N, G), (int64_t)tiled_elems(K, N, G));
-        tgroup[name] = G;
+    std::map<std::string, int> twide;           // 1: wide (32-column) tiles for the large-M GEMM
+    void add_tiled(const char* name, int K, int N, int layers, int G = 1, int wide = 0) {
+        const int64_t e = (int64_t)(wide ? tiled_elems_wide(K, N, G) : tiled_elems(K, N, G));
+        add_buf(name, layers, e, e);
+        tgroup[name] = G; twide[name] = wide;
     }
     bf16_t* TW(const char* n, int layer = 0) { const WsBuf& b = BI(n); return (bf16_t*)(ws + b.offset) + (size_t)b.ld * layer; }
 
@@ -105,16 +107,19 @@ namespace {
 
 constexpr int PATCH_LD = 640;      // 588 patch features padded to a multiple of 64
 constexpr int VHID_LD = 4352;      // 4304 padded to a multiple of 64
+constexpr int XN_LD = 2048 + 64;   // row strides that are a large power of two put every row of a K stage on the same L2 channel
+constexpr int EHID_LD = 16384 + 64;
 constexpr int64_t ATTN_PARTIAL_FLOATS = 32 * 16 * (16 * 64 * 4 + 32);   // 32 row blocks x 16 key splits of the suffix attention
 
 // Pick block tile and split-K factor from a cost model fitted to measurements on MI355X: a workgroup
 // is limited either by its MFMA work or by what one CU can pull from L2 (about 30 GB/s per CU with
 // every CU busy - the L1 miss queue bounds bytes in flight); workgroups run in rounds of 256 (one per
 // CU); every launch pays a fixed ramp; split-K adds the fp32 partial write and read.
-TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable) {
-    static const int tiles[] = {TILE_208x256, TILE_128x256, TILE_64x256};
+TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what) {
+    static const int tiles[] = {TILE_224x256, TILE_160x256, TILE_128x256, TILE_96x256, TILE_64x256};
     static const int splits[] = {1, 2, 3, 4, 6, 8};
-    if (const char* e = getenv("RTVLA_FORCE_TILE")) {
+    const char* only_for = getenv("RTVLA_FORCE_FOR");          // tuning aid: force tile / split for launches whose name contains this
+    if (const char* e = (only_for && !strstr(what, only_for)) ? nullptr : getenv("RTVLA_FORCE_TILE")) {
         TileChoice c{atoi(e), 1};
         if (const char* s = getenv("RTVLA_FORCE_SPLIT")) if (splittable) c.nsplit = atoi(s);
         return c;
@@ -126,14 +131,14 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
         const int bn = gemm_tile_bn(tile);
         const int bn16 = bn / 16 / (dual ? 2 : 1);
         const int mb = (M + bm - 1) / bm, nb = (ncols16 + bn16 - 1) / bn16;
-        const int mt = bm / 16;
+        const int mt = bm / 32;
         for (int sp : splits) {
             if (sp > 1 && !splittable) break;
             const int sps = (stages + sp - 1) / sp;
             if ((sp - 1) * sps >= stages || (sps & 1)) continue;
             const int blocks = mb * nb * sp;
             const int rounds = (blocks + 255) / 256;
-            const double mfma_us = mt * sps * 4.0 * 2 * 16 / 2400.0;
+            const double mfma_us = mt * sps * 2.0 * 4 * 32 / 2400.0;      // 32x32x16 MFMAs per wave: mt x 2 column tiles x 4 k16 steps, 32 cycles each
             const double bytes = (double)(std::min(M, bm) + bn) * sps * 64 * 2 + (splittable ? (double)std::min(M, bm) * bn * 4 : 0.0);
             double t = rounds * std::max(mfma_us, bytes / cu_bw) + 5.0;
             if (splittable) t += (double)sp * M * ncols16 * 16 * 4.0 / 4.0e6;          // the reduce pass reads the partials at ~4 TB/s
@@ -215,17 +220,17 @@ int build_tables(rtvla_ctx* c) {
     if (pi05) c->add_tensor("valid_encoder_len", false, 4, {1});
 
     // ---- workspace: re-tiled weights first, then activations ----
-    c->add_tiled("t_vision_patch_embedding_w", 588, 1152, 1, 16);
-    c->add_tiled("t_vision_attn_qkv_w", 1152, 3456, V, 16);
-    c->add_tiled("t_vision_attn_o_w", 1152, 1152, V, 16);
-    c->add_tiled("t_vision_ffn_up_w", 1152, 4304, V, 16);
-    c->add_tiled("t_vision_ffn_down_w", 4304, 1152, V, 16);
-    c->add_tiled("t_encoder_multi_modal_projector_w", 1152, 2048, 1, 16);
-    c->add_tiled("t_encoder_attn_qkv_w", 2048, 2560, L, 16);
-    c->add_tiled("t_encoder_attn_o_w", 2048, 2048, L, 16);
-    c->add_tiled("t_encoder_ffn_gate_w", 2048, 16384, L, 8);
-    c->add_tiled("t_encoder_ffn_up_w", 2048, 16384, L, 8);
-    c->add_tiled("t_encoder_ffn_down_w", 16384, 2048, L, 16);
+    c->add_tiled("t_vision_patch_embedding_w", 588, 1152, 1, 8, 1);
+    c->add_tiled("t_vision_attn_qkv_w", 1152, 3456, V, 8, 1);
+    c->add_tiled("t_vision_attn_o_w", 1152, 1152, V, 8, 1);
+    c->add_tiled("t_vision_ffn_up_w", 1152, 4304, V, 8, 1);
+    c->add_tiled("t_vision_ffn_down_w", 4304, 1152, V, 8, 1);
+    c->add_tiled("t_encoder_multi_modal_projector_w", 1152, 2048, 1, 8, 1);
+    c->add_tiled("t_encoder_attn_qkv_w", 2048, 2560, L, 8, 1);
+    c->add_tiled("t_encoder_attn_o_w", 2048, 2048, L, 8, 1);
+    c->add_tiled("t_encoder_ffn_gate_w", 2048, 16384, L, 4, 1);
+    c->add_tiled("t_encoder_ffn_up_w", 2048, 16384, L, 4, 1);
+    c->add_tiled("t_encoder_ffn_down_w", 16384, 2048, L, 8, 1);
     c->add_tiled("t_decoder_attn_qkv_w", 1024, 2560, L);
     c->add_tiled("t_decoder_attn_o_w", 2048, 1024, L);
     c->add_tiled("t_decoder_ffn_gate_w", 1024, 4096, L);
@@ -254,10 +259,10 @@ int build_tables(rtvla_ctx* c) {
     c->add_buf("vision_attn", S_v, 1152, 1152);
     c->add_buf("vision_hidden", S_v, 4304, VHID_LD);
     c->add_buf("encoder_x", S_e, 2048, 2048);
-    c->add_buf("encoder_x_norm", S_e, 2048, 2048);
+    c->add_buf("encoder_x_norm", S_e, 2048, XN_LD);
     c->add_buf("encoder_Q", ((8 * S_e + 31) / 32) * 32, 256, 256);   // fragment-tiled, rows = token*8 + head
     c->add_buf("encoder_attn", S_e, 2048, 2048);
-    c->add_buf("encoder_hidden", S_e, 16384, 16384);
+    c->add_buf("encoder_hidden", S_e, 16384, EHID_LD);
     c->add_buf("encoder_K", L * c->keys_pad, 256, 256);           // fragment-tiled [keys_pad][256] per layer
     c->add_buf("encoder_Vt", L * 256, c->keys_pad, c->keys_pad);  // tiled V^T [256][keys_pad] per layer
     c->add_buf("decoder_x", 64, 1024, 1024);                      // the decoder_* activations are fragment-tiled
@@ -289,11 +294,11 @@ struct Sched {
     Sched(rtvla_ctx* c_, hipStream_t s_) : c(c_), s(s_), d(c_->d), pi05(c_->d.model == RTVLA_PI05) {}
 
     void gemm(const bf16_t* A, int lda, int a_rows, int M, const bf16_t* B0, const bf16_t* B1, int K, int N, int epi, GemmP extra, const char* what) {
-        const int bgroup = epi == EPI_GEGLU ? 8 : 16;
+        const int bgroup = epi == EPI_GEGLU ? 4 : 8;
         GemmP p = extra;
         p.A = A; p.lda = lda; p.a_rows = a_rows; p.M = M; p.B0 = B0; p.B1 = B1;
         p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.bgroup = bgroup;
-        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU, epi == EPI_PARTIAL);
+        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU, epi == EPI_PARTIAL, what);
         p.nsplit = tc.nsplit;
         if (epi == EPI_PARTIAL) {
             p.partial = c->B<float>("splitk_partial"); p.ldp = N; p.pstride = (size_t)M * N;
@@ -347,7 +352,7 @@ struct Sched {
         if (!pi05 && d.prompt_len > 0) {
             if (c->want("prompt rows")) { launch_copy_rows(c->W("language_embeds"), 2048, c->B("encoder_x") + (size_t)S_v * 2048, 2048, d.prompt_len, 2048, s); c->note(0, "prompt rows"); }
         }
-        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, nullptr, 0, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, 0, "prefix rms0");
+        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, nullptr, 0, c->B("encoder_x_norm"), XN_LD, NORM_RMS, nullptr, nullptr, 1e-6f, 0, "prefix rms0");
     }
 
     bf16_t* Kc(int i) { return c->B("encoder_K") + (size_t)i * c->keys_pad * 256; }
@@ -357,7 +362,7 @@ struct Sched {
     void prefix_layer(int i) {
         const int S_e = c->S_e, L = d.llm_layers;
         GemmP e{}; e.rope = c->W("encoder_rope_weights"); e.q = c->B("encoder_Q"); e.k = Kc(i); e.vt = Vt(i); e.ldvt = c->keys_pad;
-        gemm(c->B("encoder_x_norm"), 2048, S_e, S_e, c->TW("t_encoder_attn_qkv_w", i), nullptr, 2048, 2560, EPI_QKV_ROPE, e, "prefix qkv");
+        gemm(c->B("encoder_x_norm"), XN_LD, S_e, S_e, c->TW("t_encoder_attn_qkv_w", i), nullptr, 2048, 2560, EPI_QKV_ROPE, e, "prefix qkv");
         if (i == L - 1) return;                      // the last layer only fills the KV cache
         AttnP a{};
         a.q = c->B("encoder_Q"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
@@ -365,11 +370,11 @@ struct Sched {
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = 0;
         if (c->want("prefix attn")) c->note(launch_mqa_attention(a, 4, s), "prefix attn");
         gemm(c->B("encoder_attn"), 2048, S_e, S_e, c->TW("t_encoder_attn_o_w", i), nullptr, 2048, 2048, EPI_PARTIAL, GemmP{}, "prefix o");
-        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix o reduce");
-        GemmP g{}; g.out = c->B("encoder_hidden"); g.ldo = 16384;
-        gemm(c->B("encoder_x_norm"), 2048, S_e, S_e, c->TW("t_encoder_ffn_gate_w", i), c->TW("t_encoder_ffn_up_w", i), 2048, 16384, EPI_GEGLU, g, "prefix geglu");
-        gemm(c->B("encoder_hidden"), 16384, S_e, S_e, c->TW("t_encoder_ffn_down_w", i), nullptr, 16384, 2048, EPI_PARTIAL, GemmP{}, "prefix down");
-        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), 2048, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix down reduce");
+        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), XN_LD, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix o reduce");
+        GemmP g{}; g.out = c->B("encoder_hidden"); g.ldo = EHID_LD;
+        gemm(c->B("encoder_x_norm"), XN_LD, S_e, S_e, c->TW("t_encoder_ffn_gate_w", i), c->TW("t_encoder_ffn_up_w", i), 2048, 16384, EPI_GEGLU, g, "prefix geglu");
+        gemm(c->B("encoder_hidden"), EHID_LD, S_e, S_e, c->TW("t_encoder_ffn_down_w", i), nullptr, 16384, 2048, EPI_PARTIAL, GemmP{}, "prefix down");
+        reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), XN_LD, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix down reduce");
     }
 
     // action-expert activations live in the fragment-tiled layout (64 rows x cols)
@@ -482,7 +487,7 @@ struct Sched {
         const int V = d.vision_layers, L = d.llm_layers;
         launch_fill_zero(c->ws + c->act_begin, c->ws_bytes - c->act_begin, s);
         auto tile = [&](const char* src, const char* dst, int K, int N, int layers) {
-            for (int i = 0; i < layers; ++i) launch_pretile(c->W(src, (size_t)K * N, i), K, N, c->TW(dst, i), c->tgroup.at(dst), s);
+            for (int i = 0; i < layers; ++i) launch_pretile(c->W(src, (size_t)K * N, i), K, N, c->TW(dst, i), c->tgroup.at(dst), c->twide.at(dst), s);
         };
         tile("vision_patch_embedding_w", "t_vision_patch_embedding_w", 588, 1152, 1);
         tile("vision_attn_qkv_w", "t_vision_attn_qkv_w", 1152, 3456, V);
@@ -511,7 +516,7 @@ struct Sched {
         launch_scale_inplace(c->B("decoder_out_proj_w_scaled"), 1024 * 32, dt, s);
         launch_copy_bytes(c->W("decoder_action_out_proj_b"), c->B("decoder_out_proj_b_scaled"), 64, s);
         launch_scale_inplace(c->B("decoder_out_proj_b_scaled"), 32, dt, s);
-        launch_pretile(c->B("decoder_out_proj_w_scaled"), 1024, 32, c->TW("t_decoder_out_proj_w"), 1, s);
+        launch_pretile(c->B("decoder_out_proj_w_scaled"), 1024, 32, c->TW("t_decoder_out_proj_w"), 1, 0, s);
         tile("decoder_time_mlp_in_w", "t_decoder_time_mlp_in_w", 1024, 1024, 1);
         tile("decoder_time_mlp_out_w", "t_decoder_time_mlp_out_w", 1024, 1024, 1);
         tile("decoder_pre_attn_norm_mod_w", "t_decoder_pre_attn_norm_mod_w", 1024, 3072, L);
@@ -769,7 +774,7 @@ size_t rtvla_pretile_elems(int K, int N) { return (K > 0 && N > 0) ? tiled_elems
 
 int rtvla_pretile(const void* w, int K, int N, void* w_tiled, void* stream) {
     if (!w || !w_tiled || K <= 0 || N <= 0) return RTVLA_ERR_ARG;
-    launch_pretile((const bf16_t*)w, K, N, (bf16_t*)w_tiled, 1, (hipStream_t)stream);
+    launch_pretile((const bf16_t*)w, K, N, (bf16_t*)w_tiled, 1, 0, (hipStream_t)stream);
     return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
 }
 
