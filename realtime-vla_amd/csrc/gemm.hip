@@ -11,6 +11,7 @@
 // every lane ends up with 4 groups of 4 consecutive output columns of one row: 8-byte packed stores,
 // and RoPE pairs / GeGLU partners sit in the same lane.
 #include "kernels.h"
+#include <algorithm>
 
 namespace {
 
@@ -86,14 +87,14 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
             ar[it] = *(const bf16x8*)(p.A + (size_t)gr * p.lda + s * 64 + kc * 8);
         }
     };
-    auto store_a = [&](int buf, bf16x8 (&ar)[AIT]) __attribute__((always_inline)) {
+    auto store_a = [&](bf16_t* buf, bf16x8 (&ar)[AIT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < AIT; ++it) {
             const int c = min(it * NTH + tid, A_CHUNKS - 1);      // duplicates write identical data
             const int row = c >> 3, kc = c & 7, ks = kc >> 1, hh = kc & 1;
             const int rr = row & 31;
             const int off = ((((row >> 5) * 4 + ks) * 64) + 8 * ((rr >> 3) + 4 * hh) + ((rr + 2 * ks + hh) & 7)) * 8;
-            *(bf16x8*)(lds + buf * STAGE_ELEMS + off) = ar[it];
+            *(bf16x8*)(buf + off) = ar[it];
         }
     };
     auto load_b_half = [&](int s, bf16x8 (&br)[NT][4], int kk) __attribute__((always_inline)) {
@@ -105,68 +106,155 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
     int lane_off[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) lane_off[ks] = (8 * ((r >> 3) + 4 * h) + ((r + 2 * ks + h) & 7)) * 8;
-    // One K stage.  Both operands are prefetched TWO stages ahead: the activations of stage t+2 go to the
-    // register set whose contents (stage t) already sit in LDS, and each half of the weight registers is
-    // re-loaded with stage t+2 as soon as the MFMAs of stage t have consumed it, so no third register set
-    // is needed.  The scheduler is given the instruction order explicitly: fragment reads run PRE ahead of
-    // the MFMAs that use them and the global loads are spread one per MFMA group.
-    auto stage = [&](int buf, int s_next, bf16x8 (&br)[NT][4], bf16x8 (&ar_next)[AIT], bf16x8 (&ar_store)[AIT]) __attribute__((always_inline)) {
-        const bf16_t* base = lds + buf * STAGE_ELEMS;
+    // One K stage, software-pipelined so that nothing but MFMAs sits on the critical path:
+    //  * LDS holds THREE stage buffers.  Stage t reads buffer `rd`; in its first half it also writes the
+    //    activations of stage t+1 into `wr`, and the single barrier of the stage sits in the MIDDLE, between
+    //    the two k halves, with MFMAs queued on both sides.  A wave that runs ahead into stage t+1 writes the
+    //    third buffer, which everybody finished reading before that barrier, so one barrier per stage is
+    //    enough, and the first fragments of stage t+1 are read before stage t ends (carried in `afn`).
+    //  * global loads run two stages ahead: the activations of stage t+2 go to the register set that was
+    //    stored to LDS during stage t-1, and each half of the weight registers is re-loaded with stage t+2 as
+    //    soon as the MFMAs of stage t have consumed it, so no third register set is needed.
+    //  * the scheduler is given the instruction order explicitly: fragment reads run PRE ahead of the MFMAs
+    //    that use them and loads / LDS writes are spread one per MFMA group.
+    constexpr int PRE = MT >= 3 ? 3 : MT;
+    constexpr int HR = 2 * MT;                                          // fragment reads per k half
+    static_assert(HR >= 2 * NT && AIT <= HR, "not enough MFMA groups to spread the loads over");
+    bf16x8 afn[PRE];                                                    // first fragments of the coming stage
+    auto frag = [&](const bf16_t* base, int f) __attribute__((always_inline)) {     // f = ks * MT + i
+        const int ks = f / MT, i = f - ks * MT;
+        return *(const bf16x8*)(base + (i * 4 + ks) * 512 + lane_off[ks]);
+    };
+    auto stage = [&](const bf16_t* rd, bf16_t* wr, int s_next, bf16x8 (&br)[NT][4], bf16x8 (&ar_next)[AIT], bf16x8 (&ar_store)[AIT]) __attribute__((always_inline)) {
+        // ---- first k half ----
         load_a(s_next, ar_next);
-        bf16x8 af[4][MT];
+        bf16x8 af[4 * MT];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
+        for (int f = 0; f < PRE; ++f) af[f] = afn[f];
 #pragma unroll
-            for (int i = 0; i < MT; ++i) af[ks][i] = *(const bf16x8*)(base + (i * 4 + ks) * 512 + lane_off[ks]);
+        for (int f = PRE; f < HR + PRE; ++f) af[f] = frag(rd, f);      // includes the first PRE fragments of the second half
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+        for (int f = 0; f < HR; ++f)
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
+            for (int j = 0; j < NT; ++j) acc[f % MT][j] = mfma32(br[j][f / MT], af[f], acc[f % MT][j]);
+        store_a(wr, ar_store);
 #pragma unroll
-                for (int j = 0; j < NT; ++j) acc[i][j] = mfma32(br[j][ks], af[ks][i], acc[i][j]);
+        for (int t = 0; t < HR; ++t) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (t < AIT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                        // activation loads of stage t+2
+            if (t >= HR - AIT) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                  // LDS writes of stage t+1
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- second k half ----
         load_b_half(s_next, br, 0);
 #pragma unroll
-        for (int ks = 2; ks < 4; ++ks)
+        for (int f = HR + PRE; f < 2 * HR; ++f) af[f] = frag(rd, f);
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
+        for (int f = 0; f < PRE; ++f) afn[f] = frag(wr, f);            // written before the barrier above
 #pragma unroll
-                for (int j = 0; j < NT; ++j) acc[i][j] = mfma32(br[j][ks], af[ks][i], acc[i][j]);
+        for (int f = HR; f < 2 * HR; ++f)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) acc[f % MT][j] = mfma32(br[j][f / MT], af[f], acc[f % MT][j]);
         load_b_half(s_next, br, 1);
-        constexpr int PRE = 3;
-        constexpr int R = 4 * MT;                                       // fragment reads of the stage
-        static_assert(R / 2 >= 2 * NT && AIT <= R / 2, "not enough MFMA groups to spread the loads over");
-        __builtin_amdgcn_sched_group_barrier(0x100, PRE, 0);
 #pragma unroll
-        for (int t = 0; t < R; ++t) {
+        for (int t = 0; t < HR; ++t) {
             __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
-            if (t < R - PRE) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (t < AIT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                        // activation loads
-            if (t >= R / 2 && t < R / 2 + 2 * NT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // weight loads, k half 0
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (t < 2 * NT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                     // weight loads, k half 0 of stage t+2
         }
         __builtin_amdgcn_sched_group_barrier(0x020, 2 * NT, 0);                                    // weight loads, k half 1
         __builtin_amdgcn_sched_barrier(0);
-        store_a(buf ^ 1, ar_store);
-        __syncthreads();
     };
 
-    // K loop, two stages per trip so the register sets and LDS buffers alternate without a runtime index and
-    // the body has a single exit.  Past the end the prefetch re-reads the last stage instead of branching.
+    // K loop, two stages per trip so the register sets alternate without a runtime index and the body has a
+    // single exit; the LDS buffers rotate through three pointers.  Past the end the prefetch re-reads the last
+    // stage instead of branching.
     const int n_st = s_end - s_begin;
     if (n_st > 0) {
         const int last = s_end - 1;
+        bf16_t* b0 = lds; bf16_t* b1 = lds + STAGE_ELEMS; bf16_t* b2 = lds + 2 * STAGE_ELEMS;
         load_a(s_begin, areg0);
         load_b_half(s_begin, breg0, 0); load_b_half(s_begin, breg0, 1);
         load_a(min(s_begin + 1, last), areg1);
         load_b_half(min(s_begin + 1, last), breg1, 0); load_b_half(min(s_begin + 1, last), breg1, 1);
-        store_a(0, areg0);
+        store_a(b0, areg0);
         __syncthreads();
+#pragma unroll
+        for (int f = 0; f < PRE; ++f) afn[f] = frag(b0, f);
         for (int s = s_begin; s < s_end; s += 2) {          // the host guarantees an even stage count per split
-            stage(0, min(s + 2, last), breg0, areg0, areg1);
-            stage(1, min(s + 3, last), breg1, areg1, areg0);
+            stage(b0, b1, min(s + 2, last), breg0, areg0, areg1);
+            stage(b1, b2, min(s + 3, last), breg1, areg1, areg0);
+            bf16_t* t0 = b0; b0 = b2; b2 = b1; b1 = t0;     // (b0, b1, b2) <- (b2, b0, b1)
         }
     }
+    __syncthreads();                                        // the epilogue reuses the stage buffers
 
     // ---- epilogue: lane (h, r) holds rows m = m0 + 32 i + r, columns n = 32 tile + 8 grp + 4 h + e ----
+    // Row-major outputs go through LDS one 32-row tile at a time so that the global stores are whole
+    // 16-byte chunks of contiguous row segments (256 B - 1 KB per row) instead of 8-byte pieces of 32 rows.
+    constexpr bool ROWMAJOR = (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_PATCH || EPI == EPI_GEGLU || EPI == EPI_PARTIAL);
+    if constexpr (ROWMAJOR) {
+        constexpr int ESZ = (EPI == EPI_PARTIAL) ? 4 : 2;
+        constexpr int OUTW = WN * HALF * 32;                       // output columns of the workgroup
+        constexpr int ROWB = OUTW * ESZ + 16;                      // padded LDS row pitch in bytes
+        constexpr int CPR = OUTW * ESZ / 16;                       // 16-byte chunks per row
+        constexpr int RPP = NTH / CPR;                             // rows per copy pass
+        static_assert(NTH % CPR == 0 && 32 % RPP == 0, "copy-out mapping");
+        unsigned char* obuf = smem_raw;
+        const int nbase = n_blk * OUTW;
+        const int ncols = p.N16 * 16;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int m = m0 + i * 32 + r;
+#pragma unroll
+            for (int j = 0; j < HALF; ++j) {
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    const int cl = (wn * HALF + j) * 32 + 8 * grp + 4 * h;        // column inside the workgroup tile
+                    const int n0 = min(nbase + cl, ncols - 4);                    // clamped: out-of-range columns are never copied out
+                    f32x4 v = {acc[i][j][4 * grp], acc[i][j][4 * grp + 1], acc[i][j][4 * grp + 2], acc[i][j][4 * grp + 3]};
+                    unsigned char* dst = obuf + r * ROWB + cl * ESZ;
+                    if constexpr (EPI == EPI_PARTIAL) {
+                        *(f32x4*)dst = v;
+                    } else if constexpr (EPI == EPI_GEGLU) {
+                        const f32x4 u = {acc[i][j + HALF][4 * grp], acc[i][j + HALF][4 * grp + 1], acc[i][j + HALF][4 * grp + 2], acc[i][j + HALF][4 * grp + 3]};
+                        *(bf16x4*)dst = pack4(gelu_tanh(v[0]) * u[0], gelu_tanh(v[1]) * u[1], gelu_tanh(v[2]) * u[2], gelu_tanh(v[3]) * u[3]);
+                    } else {
+                        const bf16x4 b = load4(p.bias + n0);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += bf2f(b[e]);
+                        if constexpr (EPI == EPI_PATCH) {
+                            const bf16x4 rs = load4(p.res + (size_t)(min(m, p.M - 1) % p.res_mod) * p.ldr + n0);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] += bf2f(rs[e]);
+                        }
+                        if constexpr (EPI == EPI_BIAS_GELU) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+                        }
+                        *(bf16x4*)dst = pack4(v);
+                    }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int ps = 0; ps < 32 / RPP; ++ps) {
+                const int row = ps * RPP + tid / CPR, ch = tid % CPR;
+                const int mm = m0 + i * 32 + row;
+                const int n = nbase + ch * (16 / ESZ);
+                if (mm < p.M && n < ncols) {
+                    const uint4 val = *(const uint4*)(obuf + row * ROWB + ch * 16);
+                    if constexpr (EPI == EPI_PARTIAL) *(uint4*)(p.partial + (size_t)split * p.pstride + (size_t)mm * p.ldp + n) = val;
+                    else *(uint4*)(p.out + (size_t)mm * p.ldo + n) = val;
+                }
+            }
+            __syncthreads();
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int m = m0 + i * 32 + r;
@@ -248,7 +336,9 @@ int launch_cfg(const GemmP& p, hipStream_t s) {
     if ((nsplit - 1) * sps >= stages_total) return 3;      // an empty split would leave its partial unwritten
     if ((sps & 1) || (stages_total & 1)) return 3;          // the kernel consumes K stages in pairs
     GemmP q = p; q.nsplit = nsplit;
-    const size_t smem = (size_t)2 * BM * 64 * sizeof(bf16_t);
+    // three K-stage buffers; the row-major epilogues stage one 32-row output tile in the same memory
+    const size_t epi_bytes = (size_t)32 * (WN * HALF * 32 * (EPI == EPI_PARTIAL ? 4 : 2) + 16);
+    const size_t smem = std::max((size_t)3 * BM * 64 * sizeof(bf16_t), epi_bytes);
     auto kern = gemm_mfma_kernel<WN, MT, NT, EPI>;
     if (smem > 65536) {
         static bool done = false;
