@@ -33,7 +33,8 @@ RTVLA_DEVICE bf16x4 pack4(f32x4 v) { return pack4(v[0], v[1], v[2], v[3]); }
 RTVLA_DEVICE bf16x4 load4(const bf16_t* p) { return *(const bf16x4*)p; }
 RTVLA_DEVICE void store4(bf16_t* p, bf16x4 v) { *(bf16x4*)p = v; }
 
-RTVLA_DEVICE float sigmoidf_fast(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// hardware reciprocal (1 ulp) instead of an IEEE division: the result is rounded to bf16 anyway
+RTVLA_DEVICE float sigmoidf_fast(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 // tanh-approximated GELU written as a * sigmoid(2 sqrt(2/pi) (a + 0.044715 a^3))
 RTVLA_DEVICE float gelu_tanh(float a) {
     return a * sigmoidf_fast(1.5957691216057308f * a * (1.0f + 0.044715f * a * a));
