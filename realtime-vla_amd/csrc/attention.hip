@@ -14,32 +14,15 @@
 //
 // The suffix pass has only ~26 row tiles but ~840 keys, and one CU can pull only ~100 GB/s through its
 // L2 port, so a workgroup that walks all keys is bound by that port.  Its keys are therefore split over
-// gridDim.y workgroups: each writes an un-normalised partial (O, row max, row sum) and takes a ticket
-// from a per-row-tile counter; the workgroup that draws the last ticket merges the partials and resets
-// the counter.  Nobody waits on anybody, so the grid always drains.  The partial records cross XCDs (each
-// has its own L2), so they are written and read with device-scope atomic accesses, which go through to the
-// memory-side coherence point: a device-scope release fence instead would write back the whole L2 once per
-// wave, which costs more than the attention itself.
+// gridDim.y workgroups, each writing an un-normalised partial (O, row max, row sum); a second small
+// kernel (attn_merge_kernel) combines the partials.  Merging inside the first kernel (last workgroup to
+// finish does it) was measured slower: the partials cross XCDs, whose L2s are not coherent with each
+// other, and device-scope fences or write-through accesses cost more than one extra launch.
 #include "kernels.h"
 
 namespace {
 
 constexpr float NEG_BIG = -1.0e30f;
-
-// device-coherent accesses to the key-split partial records
-RTVLA_DEVICE void coherent_store4(float* dst, f32x4 v) {
-    unsigned long long lo = ((unsigned long long)__float_as_uint(v[1]) << 32) | __float_as_uint(v[0]);
-    unsigned long long hi = ((unsigned long long)__float_as_uint(v[3]) << 32) | __float_as_uint(v[2]);
-    __hip_atomic_store((unsigned long long*)dst, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store((unsigned long long*)dst + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-RTVLA_DEVICE f32x4 coherent_load4(const float* src) {
-    const unsigned long long lo = __hip_atomic_load((const unsigned long long*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned long long hi = __hip_atomic_load((const unsigned long long*)src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return f32x4{__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)), __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
-}
-RTVLA_DEVICE void coherent_store(float* dst, float v) { __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-RTVLA_DEVICE float coherent_load(const float* src) { return __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 RTVLA_DEVICE bf16x8 cat44(bf16x4 lo, bf16x4 hi) {
     bf16x8 v;
@@ -209,17 +192,13 @@ void mqa_kernel(AttnP p) {
         for (int ww = 0; ww < WAVES; ++ww) lt += ls[(ww * MQ + mq) * 16 + r];
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         const int row = m0 + mq * 16 + r;
-        if (nsplit > 1 && w == 0 && g == 0) {
-            if (p.dbg & 1) { mine[mq * REC + 4096 + r] = mgl[mq]; mine[mq * REC + 4112 + r] = lt; }
-            else { coherent_store(mine + mq * REC + 4096 + r, mgl[mq]); coherent_store(mine + mq * REC + 4112 + r, lt); }
-        }
+        if (nsplit > 1 && w == 0 && g == 0) { mine[mq * REC + 4096 + r] = mgl[mq]; mine[mq * REC + 4112 + r] = lt; }
         for (int dt = w; dt < 16; dt += WAVES) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ww = 0; ww < WAVES; ++ww) t += obuf[((size_t)ww * 16 + dt) * 64 + lane];
             if (nsplit > 1) {
-                if (p.dbg & 1) *(f32x4*)(mine + mq * REC + (dt * 64 + lane) * 4) = t;
-                else coherent_store4(mine + mq * REC + (dt * 64 + lane) * 4, t);
+                *(f32x4*)(mine + mq * REC + (dt * 64 + lane) * 4) = t;
             } else if (row < p.rows) {
                 const int d = dt * 16 + 4 * g;
                 // tiled output: the [tokens][8*256] matrix the suffix O-projection reads as MFMA fragments
@@ -228,47 +207,45 @@ void mqa_kernel(AttnP p) {
             }
         }
     }
-    if (nsplit == 1 || (p.dbg & 2)) return;
+}
 
-    // ---- ticket: the last workgroup of this row block to finish merges all splits ----
-    __shared__ unsigned last_flag;
-    __builtin_amdgcn_s_waitcnt(0);             // every wave's partial stores have been acknowledged by the coherence point
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned old = __hip_atomic_fetch_add(p.counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const unsigned last = old == (unsigned)(nsplit - 1);
-        if (last) __hip_atomic_store(p.counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
-        last_flag = last;
-    }
-    __syncthreads();
-    if (!last_flag) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    const float* const all = p.partial + (size_t)blockIdx.x * nsplit * (MQ * REC);
+// Combine the key-split partials of mqa_kernel: one wave per (row block, 16-wide d tile), 4 waves per workgroup.
+// All loads of a wave are independent, so the kernel is one memory round trip long.
+template <int MQ, int NS>
+__global__ __launch_bounds__(256)
+void attn_merge_kernel(AttnP p, int nsplit) {
+    constexpr int REC = 16 * 64 * 4 + 32;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int g = lane >> 4, r = lane & 15;
+    const int rb = blockIdx.x >> 2, dt = (blockIdx.x & 3) * 4 + w;
+    const float* const all = p.partial + (size_t)rb * nsplit * (MQ * REC);
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
+        float ms[NS], ls[NS];
+        f32x4 os[NS];
+#pragma unroll
+        for (int sp = 0; sp < NS; ++sp) {
+            const float* rec = all + (size_t)min(sp, nsplit - 1) * (MQ * REC) + mq * REC;
+            ms[sp] = rec[4096 + r]; ls[sp] = rec[4112 + r];
+            os[sp] = *(const f32x4*)(rec + (dt * 64 + lane) * 4);
+        }
         float mg = NEG_BIG;
-        for (int sp = 0; sp < nsplit; ++sp) mg = fmaxf(mg, coherent_load(all + (size_t)sp * (MQ * REC) + mq * REC + 4096 + r));
+#pragma unroll
+        for (int sp = 0; sp < NS; ++sp) if (sp < nsplit) mg = fmaxf(mg, ms[sp]);
         float lt = 0.f;
-        for (int sp = 0; sp < nsplit; ++sp) {
-            const float* rec = all + (size_t)sp * (MQ * REC) + mq * REC;
-            lt += __expf(coherent_load(rec + 4096 + r) - mg) * coherent_load(rec + 4112 + r);
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sp = 0; sp < NS; ++sp) {
+            const float wgt = sp < nsplit ? __expf(ms[sp] - mg) : 0.f;
+            lt += wgt * ls[sp];
+            t += os[sp] * wgt;
         }
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-        const int row = m0 + mq * 16 + r;
-        for (int dt = w; dt < 16; dt += WAVES) {
-            f32x4 t = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-            for (int sp = 0; sp < nsplit; ++sp) {
-                const float* rec = all + (size_t)sp * (MQ * REC) + mq * REC;
-                if (p.dbg & 1) t += *(const f32x4*)(rec + (dt * 64 + lane) * 4) * __expf(coherent_load(rec + 4096 + r) - mg);
-                else t += coherent_load4(rec + (dt * 64 + lane) * 4) * __expf(coherent_load(rec + 4096 + r) - mg);
-            }
-            if (row < p.rows) {
-                const int d = dt * 16 + 4 * g;
-                bf16_t* dst = p.out_tiled ? p.out + ft_index(row >> 3, (row & 7) * 256 + d, 64) : p.out + (size_t)row * p.ldo + d;
-                store4(dst, pack4(t * inv));
-            }
+        const int row = (rb * MQ + mq) * 16 + r;
+        if (row < p.rows) {
+            const int d = dt * 16 + 4 * g;
+            bf16_t* dst = p.out_tiled ? p.out + ft_index(row >> 3, (row & 7) * 256 + d, 64) : p.out + (size_t)row * p.ldo + d;
+            store4(dst, pack4(t * inv));
         }
     }
 }
@@ -369,10 +346,12 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
     p.kb_per_split = (nkb + want - 1) / want;
     const int nsplit = (nkb + p.kb_per_split - 1) / p.kb_per_split;
     if (nsplit > 1) {
-        if (!p.partial || !p.counters) return 1;
-        if ((size_t)blocks * nsplit * MQ * (16 * 64 * 4 + 32) > p.partial_floats || blocks > p.counter_count) return 3;
+        if (!p.partial || nsplit > 16) return 1;
+        if ((size_t)blocks * nsplit * MQ * (16 * 64 * 4 + 32) > p.partial_floats) return 3;
     }
     hipLaunchKernelGGL(kern, dim3(blocks, nsplit), dim3(WAVES * 64), smem, s, p);
+    if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
+    else if (nsplit > 1) hipLaunchKernelGGL((attn_merge_kernel<MQ, 8>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 

@@ -107,11 +107,9 @@ struct AttnP {
     //   j < prefix_alloc ? j < *valid_len (or prefix_alloc if valid_len == null)
     //                    : (r >= state_rows || j == prefix_alloc)
     int prefix_alloc; const int* valid_len; int state_rows;
-    // key split over workgroups (nsplit > 1): fp32 partial records and one ticket counter per row block,
-    // counters zero before the first launch (the kernel leaves them zero)
-    int nsplit; float* partial; size_t partial_floats; unsigned* counters; int counter_count;
+    // key split over workgroups (nsplit > 1, at most 16): fp32 partial records, combined by a second launch
+    int nsplit; float* partial; size_t partial_floats;
     int kb_per_split;                // filled by the launcher
-    int dbg;
 };
 int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s);
 // SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major

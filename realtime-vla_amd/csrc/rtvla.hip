@@ -86,8 +86,8 @@ struct rtvla_ctx {
     bf16_t* TW(const char* n, int layer = 0) { const WsBuf& b = BI(n); return (bf16_t*)(ws + b.offset) + (size_t)b.ld * layer; }
 
     // suffix attention: kernel variant and key split (RTVLA_ATTN_VARIANT / RTVLA_ATTN_SPLIT override, for tuning)
-    int attn_variant = getenv("RTVLA_ATTN_VARIANT") ? atoi(getenv("RTVLA_ATTN_VARIANT")) : 8;
-    int attn_split = getenv("RTVLA_ATTN_SPLIT") ? atoi(getenv("RTVLA_ATTN_SPLIT")) : 1;
+    int attn_variant = getenv("RTVLA_ATTN_VARIANT") ? atoi(getenv("RTVLA_ATTN_VARIANT")) : 10;
+    int attn_split = getenv("RTVLA_ATTN_SPLIT") ? atoi(getenv("RTVLA_ATTN_SPLIT")) : 0;      // 0: one workgroup per 128 keys
 
     int only = -1;                 // >= 0: enqueue only the launch with this index (per-kernel timing)
     std::string last_name;
@@ -279,7 +279,6 @@ int build_tables(rtvla_ctx* c) {
     const int64_t pmax = std::max(S_v * 1152, S_e * 2048) * 8;
     c->add_buf("splitk_partial", 1, pmax, pmax, 4);
     c->add_buf("attn_partial", 1, ATTN_PARTIAL_FLOATS, ATTN_PARTIAL_FLOATS, 4);
-    c->add_buf("attn_counters", 1, 64, 64, 4);
     return 0;
 }
 
@@ -427,8 +426,7 @@ struct Sched {
         a.q = c->B("decoder_q_buf"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
         a.out = c->B("decoder_attn"); a.ldo = 256; a.out_tiled = 1; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
-        a.nsplit = c->attn_split; a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
-        a.counters = c->B<unsigned>("attn_counters"); a.counter_count = 64; a.dbg = getenv("RTVLA_ATTN_DBG") ? atoi(getenv("RTVLA_ATTN_DBG")) : 0;
+        a.nsplit = c->attn_split > 0 ? c->attn_split : std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
         if (c->want("suffix attn")) c->note(launch_mqa_attention(a, c->attn_variant, s), "suffix attn");
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
         skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
