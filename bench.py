@@ -109,7 +109,7 @@ def main():
                 "launch_ms": round(geglu_ms, 4),
                 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each calibrated on a 256 MiB copy; measured for
                 # the headline shape only (profiles/gemm_geglu_pi0_3view_p20_c50_hbm_traffic.md)
-                "traffic": 212.4e6 if args.config == "headline" else None,
+                "traffic": 212.0e6 if args.config == "headline" else None,
                 "algorithmic_bytes": 2.0 * (S_e * 2048 + 2 * 2048 * 16384 + S_e * 16384)}
     # the action-expert side: one suffix layer (5 launches) streams 18 D_L-sized weight sets per step
     layer_ms = ctx.time_stage(capi.STAGE_SUFFIX_LAYER, 3, 0, 20, stream)
