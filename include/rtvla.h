@@ -91,7 +91,17 @@ int rtvla_tensor_info(const rtvla_ctx* ctx, int index, const char** name, int32_
 
 /* Bind a caller-owned device tensor by its reference name; `bytes` must equal the tensor's size.
  * Replaces `self.weights[k].copy_(v)` (pi0_infer.py:1337-1338): the library reads the caller's
- * tensor in place.  Unknown name -> RTVLA_ERR_NAME (the reference raises KeyError). */
+ * tensor in place.  Unknown name -> RTVLA_ERR_NAME (the reference raises KeyError).
+ *
+ * Pi05 only, optional (required = 0): binding all three of
+ *   "embedding_weight"  bf16 [rows][2048]  - the embedding table (pi05_infer.py:727-746); any row count,
+ *                                            taken from `bytes`
+ *   "prompt_token_ids"  int32 [prompt_len] - the caller writes the tokenised prompt here
+ *   "rope_table"        bf16 [256 views + prompt_len + chunk][256] - the RoPE table of pi05_infer.py:655-667
+ * before rtvla_prepare moves the per-call prompt staging of pi05_infer.py:769-785, :811-822 into the
+ * forward: rows [256 views, valid_encoder_len) of encoder_x become embedding[ids] * sqrt(2048) and
+ * decoder_rope_weights becomes rope_table[valid_encoder_len - 1 ...], so a call only writes the ids,
+ * valid_encoder_len, the images and the noise. */
 int rtvla_bind(rtvla_ctx* ctx, const char* name, void* device_ptr, size_t bytes);
 
 /* Bytes of scratch the context needs (re-tiled weights, activations, KV cache), and binding of a

@@ -31,7 +31,13 @@ class Engine:
             llm_layers = int(checkpoint["encoder_attn_qkv_w"].shape[0])
         self.ctx = capi.Context(model, num_views, prompt_len, chunk_size, num_steps, vision_layers, llm_layers)
         self.weights, self.buffers = {}, {}
-        for name, elem, shape, is_weight, _ in self.ctx.tensors():
+        for name, elem, shape, is_weight, required in self.ctx.tensors():
+            if is_weight and not required:
+                # optional weights (Pi05 embedding table, ~1 GB) exist only when the checkpoint brings them
+                if name in checkpoint and name not in skip_keys:
+                    v = torch.as_tensor(checkpoint[name])
+                    self.weights[name] = torch.zeros(*v.shape, dtype=_DTYPES[elem], device=self.device)
+                continue
             # zero-initialised so that a weight the checkpoint omits (the reference leaves it
             # uninitialised, benchmark.py:9-11) can never inject NaN/Inf
             t = torch.zeros(*shape, dtype=_DTYPES[elem], device=self.device)

@@ -116,8 +116,9 @@ int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s);
 void launch_vision_attention(const bf16_t* q, const bf16_t* k, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);
 
 // ----- small helpers ------------------------------------------------------------------------
+void launch_prompt_stage(const bf16_t* emb, int vocab, const int* ids, const int* valid_len, bf16_t* x_rows, int prompt_rows, int s_v,
+                         float scale, const bf16_t* rope_full, int rope_rows, bf16_t* dec_rope, int dec_rows, hipStream_t s);
 void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hipStream_t s);
-void launch_rope_table(bf16_t* table, const int* start_minus_one_ptr, int start, int count, hipStream_t s);
 void launch_copy_rows(const bf16_t* src, int lds, bf16_t* dst, int ldd, int rows, int cols, hipStream_t s);
 void launch_fill_zero(void* p, size_t bytes, hipStream_t s);
 void launch_scale_inplace(bf16_t* p, size_t n, float f, hipStream_t s);

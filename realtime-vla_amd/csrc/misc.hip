@@ -129,24 +129,36 @@ __global__ void small_linear_kernel(const bf16_t* __restrict__ x, int ldx, const
     else out[(size_t)m * ldo + n] = f2bf(acc);
 }
 
-// RoPE table rows [cos_i, sin_i] interleaved for positions pos0 .. pos0 + count - 1, where
-// pos0 = start (+ *dyn_start if the pointer is given).  /root/reference/pi0_infer.py:1319-1335.
-__global__ void rope_table_kernel(bf16_t* __restrict__ table, const int* dyn_start, int start, int count) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= count * 128) return;
-    const int row = idx >> 7, i = idx & 127;
-    const int pos = start + row + (dyn_start ? *dyn_start : 0);
-    const float inv_freq = 1.0f / powf(10000.0f, (float)(2 * i) / 256.0f);
-    const float phase = inv_freq * (float)pos;
-    table[(size_t)row * 256 + 2 * i] = f2bf(cosf(phase));
-    table[(size_t)row * 256 + 2 * i + 1] = f2bf(sinf(phase));
-}
-
 __global__ void copy_rows_kernel(const bf16_t* __restrict__ src, int lds, bf16_t* __restrict__ dst, int ldd, int rows, int cols8) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= rows * cols8) return;
     const int r = idx / cols8, c = idx - r * cols8;
     *(uint4*)(dst + (size_t)r * ldd + c * 8) = *(const uint4*)(src + (size_t)r * lds + c * 8);
+}
+
+// Pi05 prompt staging on the device (replaces the host-side embedding lookup, scaling and RoPE slicing of
+// /root/reference/pi05_infer.py:769-785, :811-822): row i < prompt_rows of the prompt gets
+// bf16(embedding[ids[i]] * scale) when S_v + i < *valid_len (rows past the prompt keep their contents, they are
+// masked), and the decoder's RoPE rows are rope_full[*valid_len - 1 + r].  One workgroup per row.
+__global__ void prompt_stage_kernel(const bf16_t* __restrict__ emb, int vocab, const int* __restrict__ ids, const int* __restrict__ valid_len,
+                                    bf16_t* __restrict__ x_rows, int prompt_rows, int s_v, float scale,
+                                    const bf16_t* __restrict__ rope_full, int rope_rows, bf16_t* __restrict__ dec_rope, int dec_rows) {
+    const int b = blockIdx.x, tid = threadIdx.x;                    // 256 threads x 8 elements = one 2048-wide row
+    const int vl = *valid_len;
+    if (b < prompt_rows) {
+        if (s_v + b >= vl) return;
+        const int id = min(max(ids[b], 0), vocab - 1);
+        const bf16x8 v = *(const bf16x8*)(emb + (size_t)id * 2048 + tid * 8);
+        bf16x8 o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = f2bf(bf2f(v[j]) * scale);
+        *(bf16x8*)(x_rows + (size_t)b * 2048 + tid * 8) = o;
+    } else {
+        const int r = b - prompt_rows;
+        if (r >= dec_rows || tid >= 32) return;
+        const int src = min(max(vl - 1 + r, 0), rope_rows - 1);
+        *(bf16x8*)(dec_rope + (size_t)r * 256 + tid * 8) = *(const bf16x8*)(rope_full + (size_t)src * 256 + tid * 8);
+    }
 }
 
 __global__ void fill_zero_kernel(uint4* p, size_t n16) {
@@ -197,16 +209,17 @@ void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t
     hipLaunchKernelGGL(small_linear_kernel, dim3((total + 255) / 256), dim3(256), 0, s, x, ldx, W, bias, out, ldo, M, K, N, act_silu, out_tiled, out_row0);
 }
 
-void launch_rope_table(bf16_t* table, const int* dyn_start, int start, int count, hipStream_t s) {
-    const int total = count * 128;
-    hipLaunchKernelGGL(rope_table_kernel, dim3((total + 255) / 256), dim3(256), 0, s, table, dyn_start, start, count);
-}
-
 void launch_copy_rows(const bf16_t* src, int lds, bf16_t* dst, int ldd, int rows, int cols, hipStream_t s) {
     if (rows <= 0 || cols <= 0) return;
     const int cols8 = cols / 8;
     const int total = rows * cols8;
     hipLaunchKernelGGL(copy_rows_kernel, dim3((total + 255) / 256), dim3(256), 0, s, src, lds, dst, ldd, rows, cols8);
+}
+
+void launch_prompt_stage(const bf16_t* emb, int vocab, const int* ids, const int* valid_len, bf16_t* x_rows, int prompt_rows, int s_v,
+                         float scale, const bf16_t* rope_full, int rope_rows, bf16_t* dec_rope, int dec_rows, hipStream_t s) {
+    hipLaunchKernelGGL(prompt_stage_kernel, dim3(prompt_rows + dec_rows), dim3(256), 0, s, emb, vocab, ids, valid_len, x_rows, prompt_rows, s_v,
+                       scale, rope_full, rope_rows, dec_rope, dec_rows);
 }
 
 void launch_fill_zero(void* p, size_t bytes, hipStream_t s) {

@@ -217,7 +217,14 @@ int build_tables(rtvla_ctx* c) {
     c->add_tensor("diffusion_noise", false, 2, {ch, 32});
     c->add_tensor("encoder_rope_weights", false, 2, {c->S_e, 256});
     c->add_tensor("decoder_rope_weights", false, 2, {c->S_d, 256});
-    if (pi05) c->add_tensor("valid_encoder_len", false, 4, {1});
+    if (pi05) {
+        c->add_tensor("valid_encoder_len", false, 4, {1});
+        // optional device-side prompt staging: token ids -> embedding rows and decoder RoPE rows inside the graph.
+        // embedding_weight may have any number of rows (its row count is taken from the bound size).
+        c->add_tensor("embedding_weight", true, 2, {257152, 2048}); c->tensors.back().required = false;
+        c->add_tensor("prompt_token_ids", false, 4, {d.prompt_len}); c->tensors.back().required = false;
+        c->add_tensor("rope_table", false, 2, {c->S_e + ch, 256}); c->tensors.back().required = false;
+    }
 
     // ---- workspace: re-tiled weights first, then activations ----
     c->add_tiled("t_vision_patch_embedding_w", 588, 1152, 1, 8, 1);
@@ -348,6 +355,14 @@ struct Sched {
         const int S_v = c->S_v, S_e = c->S_e;
         GemmP e{}; e.out = c->B("encoder_x"); e.ldo = 2048; e.bias = c->W("encoder_multi_modal_projector_b");
         gemm(c->B("vision_x_norm"), 1152, S_v, S_v, c->TW("t_encoder_multi_modal_projector_w"), nullptr, 1152, 2048, EPI_BIAS, e, "projector");
+        if (pi05 && d.prompt_len > 0 && c->T("embedding_weight").bound && c->T("prompt_token_ids").bound && c->T("rope_table").bound) {
+            if (c->want("prompt stage")) {
+                launch_prompt_stage(c->W("embedding_weight"), (int)c->T("embedding_weight").shape[0], (const int*)c->T("prompt_token_ids").ptr, valid_len(),
+                                    c->B("encoder_x") + (size_t)S_v * 2048, d.prompt_len, S_v, 45.254833995939045f /* sqrt(2048) */,
+                                    c->W("rope_table"), S_e + d.chunk_size, c->W("decoder_rope_weights"), d.chunk_size, s);
+                c->note(0, "prompt stage");
+            }
+        }
         if (!pi05 && d.prompt_len > 0) {
             if (c->want("prompt rows")) { launch_copy_rows(c->W("language_embeds"), 2048, c->B("encoder_x") + (size_t)S_v * 2048, 2048, d.prompt_len, 2048, s); c->note(0, "prompt rows"); }
         }
@@ -610,6 +625,7 @@ int rtvla_bind(rtvla_ctx* c, const char* name, void* ptr, size_t bytes) {
     auto it = c->tindex.find(name);
     if (it == c->tindex.end()) return c->fail(RTVLA_ERR_NAME, std::string("unknown tensor: ") + name);
     Tensor& t = c->tensors[it->second];
+    if (t.name == "embedding_weight" && bytes > 0 && bytes % 4096 == 0) t.shape[0] = (int64_t)(bytes / 4096);
     if (bytes != t.bytes()) return c->fail(RTVLA_ERR_SIZE, std::string("size mismatch for ") + name + ": got " + std::to_string(bytes) + ", want " + std::to_string(t.bytes()));
     if (!ptr && bytes) return c->fail(RTVLA_ERR_ARG, std::string("null pointer for ") + name);
     if (((uintptr_t)ptr & 15) != 0) return c->fail(RTVLA_ERR_ARG, std::string("pointer not 16-byte aligned: ") + name);

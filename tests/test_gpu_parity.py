@@ -293,6 +293,34 @@ def test_forward_contract_dtypes_devices_and_aliasing():
     assert set(ck) <= set(m.weights)
 
 
+def test_pi05_device_side_prompt_equals_host_staged_prompt():
+    """Token ids staged on the device (embedding gather x sqrt(2048) and decoder RoPE rows inside the graph) give
+    bit-identical actions to the reference's host route (embeds copied into encoder_x, RoPE slice copied per call,
+    pi05_infer.py:811-822), for prompts of different length on the same instance."""
+    from pi05_infer import Pi05Inference
+    dev, views, chunk, max_len, vocab = "cuda:0", 1, 10, 12, 640
+    ck = syn.pi05_checkpoint(21, 0, dev, 1, 2, state_tokens=0)
+    del ck["language_embeds"]
+    table = syn.normal_bf16(21, "embedding_weight_small", (vocab, 2048), 0.02, dev)
+    img, _, noise = syn.observation(21, views, chunk, dev)
+    m_ids = Pi05Inference(dict(ck, embedding_weight=table), views, chunk, max_tokenize_len=max_len, discrete_state_input=False)
+    assert m_ids.device_prompt and m_ids.max_prompt_len == max_len
+    m_emb = Pi05Inference(dict(ck, language_embeds=torch.zeros(max_len, 2048, dtype=torch.bfloat16, device=dev)), views, chunk,
+                          discrete_state_input=False)
+    for n in (9, 4, 12):
+        ids = syn.randint(21, "ids%d" % n, n, vocab)
+        m_emb.weights["language_embeds"] = (table[ids.to(dev)].float() * (2048.0 ** 0.5)).to(torch.bfloat16)
+        a = m_ids.forward_ids(img, noise, ids).float().clone()
+        b = m_emb.forward(img, noise).float().clone()
+        torch.cuda.synchronize()
+        assert torch.isfinite(a).all()
+        assert torch.equal(a, b), "prompt of %d tokens: max diff %g" % (n, (a - b).abs().max().item())
+    with pytest.raises(ValueError):
+        m_ids.forward_ids(img, noise, torch.zeros(max_len + 1, dtype=torch.int64))
+    with pytest.raises(KeyError):
+        m_emb.forward_ids(img, noise, torch.zeros(3, dtype=torch.int64))
+
+
 def test_constructor_errors_match_the_reference():
     from pi0_infer import Pi0Inference
     ck = syn.pi0_checkpoint(4, 1, "cuda:0", 1, 1)
