@@ -78,7 +78,7 @@ void skinny_kernel(SkinnyP p) {
     for (int c = 0; c < NCH; ++c) {
         if (c + 1 < NCH) { load_a(c + 1, a[(c + 1) & 1]); __builtin_amdgcn_sched_barrier(0); }
         if constexpr (NORM != SN_NONE) {
-            // row sums of squares over this wave's K slice, then over the 8 waves
+            // row sums of squares over this wave's K slice
             float ss[SK_MTS];
 #pragma unroll
             for (int mt = 0; mt < SK_MTS; ++mt) {
@@ -95,6 +95,9 @@ void skinny_kernel(SkinnyP p) {
 #pragma unroll
                 for (int mt = 0; mt < SK_MTS; ++mt) ssq[w * 64 + mt * 16 + r] = ss[mt];
             }
+        }
+        if constexpr (NORM == SN_ADARMS) {
+            // adaptive RMS: x^ (1 + scale) + shift is not a row scaling, so the rows are normalised before the product
             __syncthreads();
             float f[SK_MTS];
 #pragma unroll
@@ -103,25 +106,21 @@ void skinny_kernel(SkinnyP p) {
 #pragma unroll
                 for (int ww = 0; ww < SK_WAVES; ++ww) t += ssq[ww * 64 + mt * 16 + r];
                 f[mt] = rsqrtf(t / (float)p.K + p.eps);
-                if (NORM == SN_RMS) f[mt] = round_bf16(f[mt]);      // the reference keeps the factor in bf16
             }
 #pragma unroll
             for (int i = 0; i < SK_CH; ++i) {
-                bf16x8 sc, sh;
-                if constexpr (NORM == SN_ADARMS) {
-                    sc = *(const bf16x8*)(p.style + (kb0 + i) * 32 + 8 * g);
-                    sh = *(const bf16x8*)(p.style + p.K + (kb0 + i) * 32 + 8 * g);
-                }
+                const bf16x8 sc = *(const bf16x8*)(p.style + (kb0 + i) * 32 + 8 * g);
+                const bf16x8 sh = *(const bf16x8*)(p.style + p.K + (kb0 + i) * 32 + 8 * g);
 #pragma unroll
                 for (int mt = 0; mt < SK_MTS; ++mt)
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        float x = bf2f(a[0][mt][i][j]) * f[mt];
-                        if constexpr (NORM == SN_ADARMS) x = x * (1.0f + bf2f(sc[j])) + bf2f(sh[j]);
-                        a[0][mt][i][j] = f2bf(x);
-                    }
+                    for (int j = 0; j < 8; ++j)
+                        a[0][mt][i][j] = f2bf(bf2f(a[0][mt][i][j]) * f[mt] * (1.0f + bf2f(sc[j])) + bf2f(sh[j]));
             }
         }
+        // plain RMS (no learned scale left: it is folded into the weights) is a per-row factor and is applied to
+        // the accumulator after the product, as the reference does for QKV (pi0_infer.py:1005-1015): the MFMAs
+        // start as soon as the operands arrive and the statistics ride along with the K-split reduction
 #pragma unroll
         for (int i = 0; i < SK_CH; ++i)
 #pragma unroll
@@ -147,6 +146,14 @@ void skinny_kernel(SkinnyP p) {
 #pragma unroll
         for (int ww = 0; ww < SK_WAVES; ++ww) t += red[((size_t)ww * NB * SK_MTS + nb * SK_MTS + mt) * 64 + lane];
         v[nb] = t;
+    }
+    if constexpr (NORM == SN_RMS) {
+        float t = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < SK_WAVES; ++ww) t += ssq[ww * 64 + mt * 16 + r];
+        const float f = round_bf16(rsqrtf(t / (float)p.K + p.eps));      // the reference keeps the factor in bf16
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) v[nb] *= f;
     }
     if (m >= p.M) return;
     const int n0 = tile * 16 + 4 * g;
