@@ -136,7 +136,7 @@ int rtvla_forward_stage(rtvla_ctx* ctx, int stage, int layer, int step, void* hi
 int rtvla_graph_capture(rtvla_ctx* ctx, void* hip_stream);
 int rtvla_graph_launch(rtvla_ctx* ctx, void* hip_stream);
 
-/* Number of kernel launches one forward enqueues (graph nodes). */
+/* Number of kernels the last forward (or stage) enqueued: the kernel nodes of the captured graph. */
 int rtvla_launch_count(const rtvla_ctx* ctx);
 
 /* Measurement helper (no reference counterpart): run `stage` `iters` times back to back on the

@@ -357,14 +357,16 @@ int launch_epi(const GemmP& p, int tile, hipStream_t s) {
         case TILE_128x256: return launch_cfg<4, 4, 2, EPI>(p, s);
         case TILE_96x256:  return launch_cfg<4, 3, 2, EPI>(p, s);
         case TILE_64x256:  return launch_cfg<4, 2, 2, EPI>(p, s);
+        case TILE_64x128:  if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 2, 1, EPI>(p, s); else return 2;
+        case TILE_128x128: if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 4, 1, EPI>(p, s); else return 2;
     }
     return 2;
 }
 
 }  // namespace
 
-int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {256, 224, 160, 128, 96, 64}; return v[tile]; }
-int gemm_tile_bn(int tile) { return 256; }
+int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {256, 224, 160, 128, 96, 64, 64, 128}; return v[tile]; }
+int gemm_tile_bn(int tile) { return tile >= TILE_64x128 ? 128 : 256; }
 
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {
     if (p.M <= 0 || p.N16 <= 0 || p.K32p <= 0 || (p.K32p & 1) || p.a_rows <= 0 || p.bgroup < 1) return 1;

@@ -49,7 +49,7 @@ struct GemmP {
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt;
 };
 // workgroup tile (rows x columns), 4 waves each owning 64 columns (two 32-column MFMA tiles)
-enum GemmTile { TILE_256x256 = 0, TILE_224x256, TILE_160x256, TILE_128x256, TILE_96x256, TILE_64x256, TILE_COUNT };
+enum GemmTile { TILE_256x256 = 0, TILE_224x256, TILE_160x256, TILE_128x256, TILE_96x256, TILE_64x256, TILE_64x128, TILE_128x128, TILE_COUNT };
 int gemm_tile_bm(int tile);
 int gemm_tile_bn(int tile);
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s);

@@ -52,7 +52,8 @@ struct rtvla_ctx {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     std::string err;
-    int launches = 0;
+    int launches = 0;              // scheduler launches enqueued so far (index space of rtvla_time_launch)
+    int kernels = 0;               // kernels behind them (the key-split attention is two)
     int status = 0;
 
     // ---- helpers ----
@@ -97,8 +98,8 @@ struct rtvla_ctx {
         if (!yes) ++launches;
         return yes;
     }
-    void note(int rc, const char* what) {
-        ++launches;
+    void note(int rc, const char* what, int nkernels = 1) {
+        ++launches; kernels += nkernels;
         if (rc != 0 && status == 0) { status = RTVLA_ERR_DEVICE; err = std::string("launch failed: ") + what + " (code " + std::to_string(rc) + ")"; }
     }
 };
@@ -111,12 +112,14 @@ constexpr int XN_LD = 2048 + 64;   // row strides that are a large power of two 
 constexpr int EHID_LD = 16384 + 64;
 constexpr int64_t ATTN_PARTIAL_FLOATS = 32 * 16 * (16 * 64 * 4 + 32);   // 32 row blocks x 16 key splits of the suffix attention
 
-// Pick block tile and split-K factor from a cost model fitted to measurements on MI355X: a workgroup
-// is limited either by its MFMA work or by what one CU can pull from L2 (about 30 GB/s per CU with
-// every CU busy - the L1 miss queue bounds bytes in flight); workgroups run in rounds of 256 (one per
-// CU); every launch pays a fixed ramp; split-K adds the fp32 partial write and read.
+// Pick block tile and split-K factor from a cost model fitted to measurements on MI355X.  One K stage of a
+// workgroup takes the larger of its MFMA time (32 cycles per 32x32x16 MFMA at the ~2.05 GHz the chip sustains,
+// 75 % issue efficiency) and a latency-bound load time (0.1 us + 6.7 us per MB of operands pulled by the
+// workgroup); tiles of 64 rows run two workgroups per CU, which then share the MFMA pipe but overlap
+// their load latency; all workgroups together cannot pull more than ~20 TB/s out of L2; every launch pays a
+// fixed ramp and an epilogue that grows with the tile; split-K adds the reduce pass over the fp32 partials.
 TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what) {
-    static const int tiles[] = {TILE_224x256, TILE_160x256, TILE_128x256, TILE_96x256, TILE_64x256};
+    static const int tiles[] = {TILE_224x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};   // 96x256 never won a sweep
     static const int splits[] = {1, 2, 3, 4, 6, 8};
     const char* only_for = getenv("RTVLA_FORCE_FOR");          // tuning aid: force tile / split for launches whose name contains this
     if (const char* e = (only_for && !strstr(what, only_for)) ? nullptr : getenv("RTVLA_FORCE_TILE")) {
@@ -124,27 +127,35 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
         if (const char* s = getenv("RTVLA_FORCE_SPLIT")) if (splittable) c.nsplit = atoi(s);
         return c;
     }
-    const double cu_bw = 30.0e3;           // bytes per microsecond per CU
     double best = 1e30; TileChoice bc{TILE_128x256, 1};
     for (int tile : tiles) {
         const int bm = gemm_tile_bm(tile);
         const int bn = gemm_tile_bn(tile);
+        if (dual && bn < 256) continue;
         const int bn16 = bn / 16 / (dual ? 2 : 1);
         const int mb = (M + bm - 1) / bm, nb = (ncols16 + bn16 - 1) / bn16;
-        const int mt = bm / 32;
+        const int mt = bm / 32, nt = bn / 128;
+        if (!dual && tile == TILE_64x256) continue;        // measured: 64x128 is never slower than 64x256 for the single-weight GEMMs
+        const int occ = bm <= 64 ? 2 : 1;
         for (int sp : splits) {
             if (sp > 1 && !splittable) break;
             const int sps = (stages + sp - 1) / sp;
             if ((sp - 1) * sps >= stages || (sps & 1)) continue;
             const int blocks = mb * nb * sp;
-            const int rounds = (blocks + 255) / 256;
-            const double mfma_us = mt * sps * 2.0 * 4 * 32 / 2400.0;      // 32x32x16 MFMAs per wave: mt x 2 column tiles x 4 k16 steps, 32 cycles each
-            const double bytes = (double)(std::min(M, bm) + bn) * sps * 64 * 2 + (splittable ? (double)std::min(M, bm) * bn * 4 : 0.0);
-            double t = rounds * std::max(mfma_us, bytes / cu_bw) + 5.0;
-            if (splittable) t += (double)sp * M * ncols16 * 16 * 4.0 / 4.0e6;          // the reduce pass reads the partials at ~4 TB/s
+            const int per_cu = (blocks + 255) / 256;
+            const int together = std::min(occ, per_cu);
+            const int rounds = (per_cu + occ - 1) / occ;
+            const double mfma_us = mt * nt * 4 * 32 / 2050.0 / 0.75;
+            const double stage_bytes = (double)(bm + bn) * 64 * 2;
+            const double stage_us = std::max(together * mfma_us, 0.1 + stage_bytes / 1.5e5);
+            double t = std::max(rounds * sps * stage_us, blocks * (double)sps * stage_bytes / 20.0e6);
+            t += 3.5 + 2.0 + 1.2 * mt * (splittable ? 1.5 : 1.0);
+            if (splittable) t += 3.5 + (double)sp * M * ncols16 * 16 * 4.0 / 4.0e6;    // the reduce pass reads the partials at ~4 TB/s
             if (t < best) { best = t; bc = TileChoice{tile, sp}; }
         }
     }
+    if (getenv("RTVLA_PRINT_TILES")) fprintf(stderr, "rtvla tile choice: %-18s M=%d N=%d stages=%d -> %dx%d split %d (model %.1f us)\n", what, M, ncols16 * 16,
+                                             stages, gemm_tile_bm(bc.tile), gemm_tile_bn(bc.tile), bc.nsplit, best);
     return bc;
 }
 
@@ -442,7 +453,7 @@ struct Sched {
         a.out = c->B("decoder_attn"); a.ldo = 256; a.out_tiled = 1; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
         a.nsplit = c->attn_split > 0 ? c->attn_split : std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
-        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, c->attn_variant, s), "suffix attn");
+        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, c->attn_variant, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
         skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
         SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 4096;
@@ -661,7 +672,7 @@ int rtvla_buffer_info(const rtvla_ctx* c, int index, const char** name, size_t* 
 
 int rtvla_prepare(rtvla_ctx* c, void* stream) {
     if (int rc = check_ready(c, false)) return rc;
-    c->status = 0; c->launches = 0;
+    c->status = 0; c->launches = 0; c->kernels = 0;
     Sched(c, (hipStream_t)stream).prepare();
     if (c->status) return c->status;
     hipError_t e = hipGetLastError();
@@ -672,14 +683,14 @@ int rtvla_prepare(rtvla_ctx* c, void* stream) {
 
 int rtvla_forward(rtvla_ctx* c, void* stream) {
     if (int rc = check_ready(c, true)) return rc;
-    c->status = 0; c->launches = 0;
+    c->status = 0; c->launches = 0; c->kernels = 0;
     Sched(c, (hipStream_t)stream).forward();
     return c->status;
 }
 
 int rtvla_forward_stage(rtvla_ctx* c, int stage, int layer, int step, void* stream) {
     if (int rc = check_ready(c, true)) return rc;
-    c->status = 0; c->launches = 0;
+    c->status = 0; c->launches = 0; c->kernels = 0;
     int rc = Sched(c, (hipStream_t)stream).stage(stage, layer, step);
     if (rc) return c->fail(rc, "bad stage / layer / step");
     return c->status;
@@ -696,7 +707,7 @@ int rtvla_graph_capture(rtvla_ctx* c, void* stream) {
     if (c->graph) { hipGraphDestroy(c->graph); c->graph = nullptr; }
     e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) return hip_fail(c, e, "hipStreamBeginCapture");
-    c->status = 0; c->launches = 0;
+    c->status = 0; c->launches = 0; c->kernels = 0;
     Sched(c, s).forward();
     e = hipStreamEndCapture(s, &c->graph);
     if (e != hipSuccess) return hip_fail(c, e, "hipStreamEndCapture");
@@ -714,7 +725,7 @@ int rtvla_graph_launch(rtvla_ctx* c, void* stream) {
     return RTVLA_OK;
 }
 
-int rtvla_launch_count(const rtvla_ctx* c) { return c ? c->launches : 0; }
+int rtvla_launch_count(const rtvla_ctx* c) { return c ? c->kernels : 0; }
 
 int rtvla_time_stage(rtvla_ctx* c, int stage, int layer, int step, int iters, void* stream, float* mean_ms) {
     if (int rc = check_ready(c, true)) return rc;
@@ -747,12 +758,12 @@ int rtvla_time_launch(rtvla_ctx* c, int stage, int layer, int step, int launch_i
     if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
     Sched sc(c, s);
     c->status = 0; c->only = launch_index; c->last_name.clear();
-    c->launches = 0;
+    c->launches = 0; c->kernels = 0;
     int rc = sc.stage(stage, layer, step);      // warm-up, also tells whether the index exists
     if (!rc && c->launches <= launch_index) rc = c->fail(RTVLA_ERR_ARG, "launch index past the end of the stage");
     if (!rc) {
         hipEventRecord(a, s);
-        for (int i = 0; i < iters && !rc; ++i) { c->launches = 0; rc = sc.stage(stage, layer, step); }
+        for (int i = 0; i < iters && !rc; ++i) { c->launches = 0; c->kernels = 0; rc = sc.stage(stage, layer, step); }
         hipEventRecord(b, s);
         hipError_t e = hipEventSynchronize(b);
         if (e != hipSuccess) rc = hip_fail(c, e, "time_launch");
