@@ -161,6 +161,32 @@ int rtvla_time_forward(rtvla_ctx* ctx, int iters, void* hip_stream, float* ms_ou
 size_t rtvla_pretile_elems(int K, int N);
 int rtvla_pretile(const void* w, int K, int N, void* w_tiled, void* hip_stream);
 
+/* ---- observation pre-/post-processing either side of the forward (context-free, capturable) ----------------
+ * The reference does these on the host per observation (test.py:88-201).  All pointers are device pointers. */
+
+/* Replaces _resize_with_pad + _normalize_image (test.py:104-119) for one uint8 HWC RGB image: aspect-preserving
+ * bilinear resize that matches Pillow's Image.resize(BILINEAR) bit for bit, pasted centred on a black 224x224
+ * canvas, then x / 255 * 2 - 1, written as bf16 [224][224][3] - i.e. straight into one view of
+ * observation_images_normalized.  `scratch` holds the 8-bit intermediate of the horizontal pass
+ * (rtvla_preprocess_image_scratch bytes).  RTVLA_ERR_LIMIT for shrink factors above 31. */
+size_t rtvla_preprocess_image_scratch(int height, int width);
+int rtvla_preprocess_image(const void* src_u8, int height, int width, void* dst_bf16, void* scratch, size_t scratch_bytes,
+                           void* hip_stream);
+
+/* Replaces _normalize_state (+ _digitize_state) (test.py:121-137): state[n] and the statistics [n_stats] are
+ * zero-padded to 32 like _pad_to_dim; mode 0 (Pi0): (x - a) / (b + 1e-6) with a = mean, b = std; mode 1 (Pi05):
+ * (x - a) / (b - a + 1e-6) * 2 - 1 with a = q01, b = q99, all in double as numpy computes it.  Outputs (each may
+ * be null): the value as float32 -> bf16 [32] (= observation_state_normalized), as double [32], and its 256-bin
+ * index np.digitize(z, linspace(-1, 1, 257)[:-1]) - 1 as int32 [32]. */
+int rtvla_preprocess_state(const double* state, int n, const double* stat_a, const double* stat_b, int n_stats, int mode,
+                           void* out_bf16, double* out_f64, int32_t* out_bins, void* hip_stream);
+
+/* Replaces _unnormalize_actions and the delta-to-absolute step of infer (test.py:139-151, :196-201): bf16 actions
+ * [chunk][32] -> float32 -> (mode 0) x * (b + 1e-6) + a or (mode 1) (x + 1) / 2 * (b - a + 1e-6) + a in double, first
+ * action_dim columns, + ori_state, with the state taken off again on every 7th column.  out: double [chunk][action_dim]. */
+int rtvla_postprocess_actions(const void* actions_bf16, int chunk, const double* stat_a, const double* stat_b, int n_stats,
+                              int mode, const double* ori_state, int action_dim, double* out, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

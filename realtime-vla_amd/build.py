@@ -7,7 +7,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librtvla.so")
-SOURCES = ["gemm.hip", "skinny.hip", "attention.hip", "misc.hip", "rtvla.hip"]
+SOURCES = ["gemm.hip", "skinny.hip", "attention.hip", "misc.hip", "rtvla.hip", "transforms.hip"]
+# bit-exact parity with host arithmetic (Pillow, numpy): no fused multiply-adds in these files
+EXTRA = {"transforms.hip": ["-ffp-contract=off"]}
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-unused-value",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -21,7 +23,7 @@ def _hipcc():
 
 def _compile(src):
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [_hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc()] + FLAGS + EXTRA.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "warnings generated" not in l)
     if r.returncode != 0:

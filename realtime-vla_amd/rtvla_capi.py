@@ -59,6 +59,10 @@ SYMBOLS = {
     "rtvla_time_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.POINTER(ctypes.c_float)]),
     "rtvla_pretile_elems": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "rtvla_pretile": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P]),
+    "rtvla_preprocess_image_scratch": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
+    "rtvla_preprocess_image": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P, ctypes.c_size_t, _P]),
+    "rtvla_preprocess_state": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, ctypes.c_int, ctypes.c_int, _P, _P, _P, _P]),
+    "rtvla_postprocess_actions": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, ctypes.c_int, ctypes.c_int, _P, ctypes.c_int, _P, _P]),
 }
 
 _lib = None
