@@ -30,6 +30,67 @@ HBM_PEAK_GBS = 8000.0
 COPY_PROBE_BYTES = 256 << 20   # size of the calibration copy of --traffic-probe
 
 
+def bench_transforms(args, dev):
+    """One observation's pre- and post-processing: 3 uint8 frames of 480x640 already in HBM -> bf16 model buffers, raw
+    state -> normalised state, bf16 actions -> absolute float64 actions.  CPU baseline: the same steps as the reference
+    runs them (Pillow + numpy on the host, /root/reference/test.py:88-201), via the oracle's restatement."""
+    import numpy as np
+    import torch
+    from obs_transforms import ObservationTransforms
+    rng = np.random.RandomState(0)
+    frames = [rng.randint(0, 256, size=(480, 640, 3)).astype(np.uint8) for _ in range(3)]
+    stats = {g: {"mean": rng.randn(7).tolist(), "std": (rng.rand(7) + 0.5).tolist()} for g in ("state", "actions")}
+    tr = ObservationTransforms("pi0", stats, state_len=7, action_dim=7)
+    dframes = [torch.from_numpy(f).to(dev) for f in frames]
+    out = torch.empty(3, 224, 224, 3, dtype=torch.bfloat16, device=dev)
+    sbuf = torch.empty(32, dtype=torch.bfloat16, device=dev)
+    actions = torch.randn(50, 32, device=dev).to(torch.bfloat16)
+    state = rng.randn(7)
+
+    def step():
+        for v in range(3):
+            tr.resize_pad_normalize_into(dframes[v], out[v])
+        tr._normalize_state(state, out_bf16=sbuf)
+        return tr.postprocess_actions(actions, state)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(args.steps):
+        torch.cuda.synchronize(); t0 = time.perf_counter(); step(); torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e6)
+    times.sort()
+    # kernel time alone (HIP events around the three image launches)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        for v in range(3):
+            tr.resize_pad_normalize_into(dframes[v], out[v])
+    e1.record(); torch.cuda.synchronize()
+    img_us = e0.elapsed_time(e1) * 1e3 / 20
+    alg_bytes = 3 * (480 * 640 * 3 + 2 * 480 * 224 * 3 + 224 * 224 * 3 * 2)        # frame read, 8-bit intermediate write+read, bf16 write
+    result = {"metric": "us per observation pre+post-processing (3 frames 480x640 -> 224x224 bf16, state, 50x7 actions)",
+              "value": round(times[len(times) // 2], 1), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "higher_is_better": False, "dtype": "u8/f64", "data": "synthetic",
+              "roofline": {"bound": "hbm", "kernel": "resample_h_kernel + resample_v_pad_norm_kernel x 3 frames", "achieved": round(alg_bytes / img_us / 1e3, 2),
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_bytes / img_us / 1e3 / HBM_PEAK_GBS, 5), "launch_ms": round(img_us / 1e3, 4),
+                           "traffic": None}}
+    if not args.no_cpu:
+        from oracle import transforms as T
+        from PIL import Image
+        t0 = time.perf_counter()
+        for _ in range(20):
+            for f in frames:                                     # the reference's own recipe: Pillow resize + numpy
+                pil = Image.fromarray(f).resize((224, 168), resample=Image.BILINEAR)
+                canvas = Image.new(pil.mode, (224, 224), 0); canvas.paste(pil, (0, 28))
+                T.normalize_image(np.array(canvas))
+            T.normalize_state(state, stats["state"], "pi0")
+            T.postprocess_actions(actions.cpu().float().numpy(), stats["actions"], "pi0", state, 7)
+        result["cpu_baseline"] = {"value": round((time.perf_counter() - t0) / 20 * 1e6, 1), "unit": "us", "cores": 1, "kind": "port",
+                                  "sample": "20 observations, Pillow resize + numpy on one host core"}
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -37,6 +98,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    ap.add_argument("--transforms", action="store_true",
+                    help="measure the observation pre-/post-processing kernels (3 camera frames of 480x640, state, actions) instead of the forward")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: launch the roofline kernel a few times, then a "
                          "plain 256 MiB device copy whose counter reading calibrates the unit, and exit")
@@ -53,6 +116,8 @@ def main():
     model_name, views, prompt, chunk, state_tokens, desc = CONFIGS[args.config]
     dev = "cuda:0"
     seed = 1234
+    if args.transforms:
+        return bench_transforms(args, dev)
     if model_name == "pi0":
         from pi0_infer import Pi0Inference
         ck = syn.pi0_checkpoint(seed, prompt, device=dev)
