@@ -29,7 +29,7 @@ __global__ void pretile_kernel(const bf16_t* __restrict__ W, int K, int N, bf16_
 // One workgroup per row: x = bf16(res + bias + sum_s partial[s]); optional normalised copy.
 // Replaces merge_split_k_bias_res + layer_norm_small_kernel / rms_norm_kernel
 // (/root/reference/pi0_infer.py:325-346, :366-382, :648-663).
-template <int NORM>
+template <int NORM, int NSPLIT>
 __global__ __launch_bounds__(256)
 void reduce_kernel(ReduceP p) {
     __shared__ float red[8];
@@ -44,9 +44,13 @@ void reduce_kernel(ReduceP p) {
         v[it] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (c < nq) {
             const int n0 = c * 4;
+            // the split count is a template argument so that every partial is requested before the first add
+            f32x4 part[NSPLIT > 0 ? NSPLIT : 1];
+#pragma unroll
+            for (int sp = 0; sp < NSPLIT; ++sp) part[sp] = *(const f32x4*)(p.partial + (size_t)sp * p.pstride + (size_t)m * p.ldp + n0);
             f32x4 a = {0.f, 0.f, 0.f, 0.f};
-            for (int sp = 0; sp < p.nsplit; ++sp)
-                a += *(const f32x4*)(p.partial + (size_t)sp * p.pstride + (size_t)m * p.ldp + n0);
+#pragma unroll
+            for (int sp = 0; sp < NSPLIT; ++sp) a += part[sp];
             if (p.bias) { const bf16x4 b = load4(p.bias + n0); for (int e = 0; e < 4; ++e) a[e] += bf2f(b[e]); }
             if (p.res) { const bf16x4 rr = load4(p.res + (size_t)m * p.ldr + n0); for (int e = 0; e < 4; ++e) a[e] += bf2f(rr[e]); }
             const bf16x4 xb = pack4(a);
@@ -123,7 +127,19 @@ __global__ void small_linear_kernel(const bf16_t* __restrict__ x, int ldx, const
     if (idx >= M * N) return;
     const int m = idx / N, n = idx - m * N;
     float acc = bias ? bf2f(bias[n]) : 0.f;
-    for (int k = 0; k < K; ++k) acc += bf2f(x[(size_t)m * ldx + k]) * bf2f(W[(size_t)k * N + n]);
+    if (K == 32) {
+        // every operand is requested before the first use: a dependent load per k would cost 32 memory round trips
+        bf16x8 xr[4];
+        bf16_t wc[32];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xr[q] = *(const bf16x8*)(x + (size_t)m * ldx + q * 8);
+#pragma unroll
+        for (int k = 0; k < 32; ++k) wc[k] = W[(size_t)k * N + n];
+#pragma unroll
+        for (int k = 0; k < 32; ++k) acc += bf2f(xr[k >> 3][k & 7]) * bf2f(wc[k]);
+    } else {
+        for (int k = 0; k < K; ++k) acc += bf2f(x[(size_t)m * ldx + k]) * bf2f(W[(size_t)k * N + n]);
+    }
     if (act_silu) acc = siluf(acc);
     if (out_tiled) out[ft_index(m + out_row0, n, ldo >> 5)] = f2bf(acc);
     else out[(size_t)m * ldo + n] = f2bf(acc);
@@ -184,17 +200,32 @@ void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide,
     hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, KBp, G, wide, chunks);
 }
 
+template <int NORM>
+static int launch_reduce_norm(const ReduceP& p, hipStream_t s) {
+    const dim3 grid(p.M), block(256);
+    switch (p.nsplit) {
+        case 0: hipLaunchKernelGGL((reduce_kernel<NORM, 0>), grid, block, 0, s, p); break;
+        case 1: hipLaunchKernelGGL((reduce_kernel<NORM, 1>), grid, block, 0, s, p); break;
+        case 2: hipLaunchKernelGGL((reduce_kernel<NORM, 2>), grid, block, 0, s, p); break;
+        case 3: hipLaunchKernelGGL((reduce_kernel<NORM, 3>), grid, block, 0, s, p); break;
+        case 4: hipLaunchKernelGGL((reduce_kernel<NORM, 4>), grid, block, 0, s, p); break;
+        case 6: hipLaunchKernelGGL((reduce_kernel<NORM, 6>), grid, block, 0, s, p); break;
+        case 8: hipLaunchKernelGGL((reduce_kernel<NORM, 8>), grid, block, 0, s, p); break;
+        default: return 2;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 5;
+}
+
 int launch_reduce(const ReduceP& p, hipStream_t s) {
     if (p.M <= 0 || p.N <= 0 || (p.N & 3) || p.N > 2048) return 1;
     if (p.norm != NORM_NONE && !p.xn) return 1;
     if (p.norm == NORM_LAYER && (!p.nw || !p.nb)) return 1;
     switch (p.norm) {
-        case NORM_NONE:  hipLaunchKernelGGL(reduce_kernel<NORM_NONE>, dim3(p.M), dim3(256), 0, s, p); break;
-        case NORM_RMS:   hipLaunchKernelGGL(reduce_kernel<NORM_RMS>, dim3(p.M), dim3(256), 0, s, p); break;
-        case NORM_LAYER: hipLaunchKernelGGL(reduce_kernel<NORM_LAYER>, dim3(p.M), dim3(256), 0, s, p); break;
-        default: return 2;
+        case NORM_NONE:  return launch_reduce_norm<NORM_NONE>(p, s);
+        case NORM_RMS:   return launch_reduce_norm<NORM_RMS>(p, s);
+        case NORM_LAYER: return launch_reduce_norm<NORM_LAYER>(p, s);
     }
-    return hipGetLastError() == hipSuccess ? 0 : 5;
+    return 2;
 }
 
 void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hipStream_t s) {
