@@ -170,8 +170,9 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
     };
 
     // K loop, two stages per trip so the register sets alternate without a runtime index and the body has a
-    // single exit; the LDS buffers rotate through three pointers.  Past the end the prefetch re-reads the last
-    // stage instead of branching.
+    // single exit; for the tiles of at most 128 rows an odd stage count ends in one peeled stage (the larger ones
+    // need an even count).  The LDS buffers rotate through three
+    // pointers.  Past the end the prefetch re-reads the last stage instead of branching.
     const int n_st = s_end - s_begin;
     if (n_st > 0) {
         const int last = s_end - 1;
@@ -184,10 +185,14 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         __syncthreads();
 #pragma unroll
         for (int f = 0; f < PRE; ++f) afn[f] = frag(b0, f);
-        for (int s = s_begin; s < s_end; s += 2) {          // the host guarantees an even stage count per split
+        int s = s_begin;
+        for (; s + 1 < s_end; s += 2) {
             stage(b0, b1, min(s + 2, last), breg0, areg0, areg1);
             stage(b1, b2, min(s + 3, last), breg1, areg1, areg0);
             bf16_t* t0 = b0; b0 = b2; b2 = b1; b1 = t0;     // (b0, b1, b2) <- (b2, b0, b1)
+        }
+        if constexpr (MT <= 4) {                            // (the large tiles have no registers to spare for a third copy of the stage)
+            if (s < s_end) stage(b0, b1, last, breg0, areg0, areg1);
         }
     }
     __syncthreads();                                        // the epilogue reuses the stage buffers
@@ -334,7 +339,7 @@ int launch_cfg(const GemmP& p, hipStream_t s) {
     const int nsplit = p.nsplit < 1 ? 1 : p.nsplit;
     const int sps = (stages_total + nsplit - 1) / nsplit;
     if ((nsplit - 1) * sps >= stages_total) return 3;      // an empty split would leave its partial unwritten
-    if ((sps & 1) || (stages_total & 1)) return 3;          // the kernel consumes K stages in pairs
+    if (MT > 4 && ((sps & 1) || (stages_total & 1))) return 3;              // the large tiles consume K stages in pairs
     GemmP q = p; q.nsplit = nsplit;
     // three K-stage buffers; the row-major epilogues stage one 32-row output tile in the same memory
     const size_t epi_bytes = (size_t)32 * (WN * HALF * 32 * (EPI == EPI_PARTIAL ? 4 : 2) + 16);

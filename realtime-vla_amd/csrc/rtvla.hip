@@ -140,7 +140,9 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
         for (int sp : splits) {
             if (sp > 1 && !splittable) break;
             const int sps = (stages + sp - 1) / sp;
-            if ((sp - 1) * sps >= stages || (sps & 1)) continue;
+            if ((sp - 1) * sps >= stages) continue;
+            const int tail = stages - (sp - 1) * sps;                   // stages of the last split
+            if (bm > 128 && ((sps & 1) || (tail & 1))) continue;          // the large tiles consume K stages in pairs
             const int blocks = mb * nb * sp;
             const int per_cu = (blocks + 255) / 256;
             const int together = std::min(occ, per_cu);
