@@ -235,6 +235,19 @@ def test_pi0_two_views_ragged_prefix():
     check_case(Case("pi0", 21, 2, 7, 17, 1, 2))
 
 
+@pytest.mark.parametrize("model,views,prompt,chunk,state_tokens", [
+    ("pi0", 1, 1, 1, 0),        # one action row, one prompt token: 258 prefix rows, 2 suffix rows
+    ("pi0", 3, 37, 33, 0),      # odd everything: 805 prefix rows (GEMM row tiles with a ragged tail), 34 suffix rows
+    ("pi0", 2, 200, 50, 0),     # long prompt on two views: 712 prefix rows, 763 keys (6 key splits)
+    ("pi05", 2, 5, 64, 9),      # Pi05 at the 64-row limit of the action-expert tile
+    ("pi05", 3, 100, 7, 0),     # Pi05, long prompt, short chunk
+])
+def test_shape_sweep_against_the_oracle(model, views, prompt, chunk, state_tokens):
+    """Shapes between and beyond the BASELINE configurations at reduced depth: every tile choice, split count and
+    ragged tail they select must still agree with the oracle (and replay must equal the eager run)."""
+    check_case(Case(model, 100 + views * 7 + prompt, views, prompt, chunk, 1, 2, state_tokens=state_tokens))
+
+
 @pytest.mark.parametrize("name,spec", [
     ("c1", ("pi0", 1234, 1, 0, 50)),
     ("c2", ("pi0", 1234, 2, 20, 50)),
