@@ -141,13 +141,16 @@ int rtvla_launch_count(const rtvla_ctx* ctx);
 
 /* Measurement helper (no reference counterpart): run `stage` `iters` times back to back on the
  * stream between two HIP events recorded on that same stream and return the mean milliseconds
- * per run.  Synchronises the stream. */
+ * per run.  With layer = -1 every layer of the stage runs in turn (weights cold, as inside a forward) and the
+ * mean is per layer.  Synchronises the stream. */
 int rtvla_time_stage(rtvla_ctx* ctx, int stage, int layer, int step, int iters, void* hip_stream, float* mean_ms);
 
 /* Measurement helper (no reference counterpart): as rtvla_time_stage, but enqueue only the
  * `launch_index`-th kernel launch of the stage (0-based, in schedule order), so that one kernel's
  * mean duration is measured live with HIP events on the stream it is launched on.  The launch's
- * name is copied to name_out.  Returns RTVLA_ERR_ARG when the stage has fewer launches. */
+ * name is copied to name_out.  Returns RTVLA_ERR_ARG when the stage has fewer launches.  With layer = -1 the
+ * launch is enqueued once per layer in turn (per iteration), so every launch streams weights that nothing has
+ * touched since the previous pass - the condition it meets inside a forward; a fixed layer measures it cache-warm. */
 int rtvla_time_launch(rtvla_ctx* ctx, int stage, int layer, int step, int launch_index, int iters, void* hip_stream,
                       float* mean_ms, char* name_out, size_t name_cap);
 

@@ -737,14 +737,20 @@ int rtvla_time_stage(rtvla_ctx* c, int stage, int layer, int step, int iters, vo
     if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
     Sched sc(c, s);
     c->status = 0;
-    int rc = sc.stage(stage, layer, step);      // warm-up
+    // layer -1: every layer of the stage in turn (weights cold, as inside a forward), mean per layer
+    const bool cycle = layer == -1;
+    const int n_layers = !cycle ? 1 : (stage == RTVLA_STAGE_VISION_LAYER ? c->d.vision_layers :
+                                       (stage == RTVLA_STAGE_PREFIX_LAYER || stage == RTVLA_STAGE_SUFFIX_LAYER) ? c->d.llm_layers : 1);
+    const int first = cycle ? 0 : layer;
+    int rc = sc.stage(stage, first, step);      // warm-up
     if (!rc) {
         hipEventRecord(a, s);
-        for (int i = 0; i < iters && !rc; ++i) rc = sc.stage(stage, layer, step);
+        for (int i = 0; i < iters && !rc; ++i)
+            for (int l = first; l < first + n_layers && !rc; ++l) rc = sc.stage(stage, l, step);
         hipEventRecord(b, s);
         hipError_t e = hipEventSynchronize(b);
         if (e != hipSuccess) rc = hip_fail(c, e, "time_stage");
-        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / iters; }
+        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / (iters * n_layers); }
     }
     hipEventDestroy(a); hipEventDestroy(b);
     if (rc) return rc;
@@ -761,15 +767,27 @@ int rtvla_time_launch(rtvla_ctx* c, int stage, int layer, int step, int launch_i
     Sched sc(c, s);
     c->status = 0; c->only = launch_index; c->last_name.clear();
     c->launches = 0; c->kernels = 0;
-    int rc = sc.stage(stage, layer, step);      // warm-up, also tells whether the index exists
+    // layer -1: one launch per layer in turn, so that every launch streams weights nobody has touched since the
+    // previous pass (what the kernel sees inside a forward); otherwise the same layer over and over (cache-warm)
+    const bool cycle = layer == -1;
+    const int n_layers = !cycle ? 1 : (stage == RTVLA_STAGE_VISION_LAYER ? c->d.vision_layers :
+                                       (stage == RTVLA_STAGE_PREFIX_LAYER || stage == RTVLA_STAGE_SUFFIX_LAYER) ? c->d.llm_layers : 1);
+    const int first = cycle ? 0 : layer;
+    int rc = sc.stage(stage, first, step);      // warm-up, also tells whether the index exists
     if (!rc && c->launches <= launch_index) rc = c->fail(RTVLA_ERR_ARG, "launch index past the end of the stage");
     if (!rc) {
+        int enqueued = 0;
         hipEventRecord(a, s);
-        for (int i = 0; i < iters && !rc; ++i) { c->launches = 0; c->kernels = 0; rc = sc.stage(stage, layer, step); }
+        for (int i = 0; i < iters && !rc; ++i)
+            for (int l = first; l < first + n_layers && !rc; ++l) {
+                c->launches = 0; c->kernels = 0;
+                rc = sc.stage(stage, l, step);
+                enqueued += c->launches > launch_index;          // (the last prefix layer has fewer launches)
+            }
         hipEventRecord(b, s);
         hipError_t e = hipEventSynchronize(b);
         if (e != hipSuccess) rc = hip_fail(c, e, "time_launch");
-        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / iters; }
+        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / (enqueued > 0 ? enqueued : 1); }
     }
     c->only = -1;
     hipEventDestroy(a); hipEventDestroy(b);
