@@ -71,6 +71,22 @@ void skinny_kernel(SkinnyP p) {
             for (int i = 0; i < SK_CH; ++i) dst[mt][i] = *(const bf16x8*)(arow[mt] + (c * SK_CH + i) * astep);
     };
     load_a(0, a[0]);
+    // what the epilogue will need from memory (old residual, RoPE pair, bias, gate) is requested now as well, by the
+    // waves that will finish a row tile, so that no memory round trip is left after the reduction
+    bf16x4 pre_old = {}, pre_cs = {}, pre_bias = {}, pre_gate = {};
+    if (w < SK_MTS) {
+        const int me = min(m_base + w * 16 + r, p.M - 1);
+        const int ne = tile * 16 + 4 * g;
+        if constexpr (EPI == SK_RES) {
+            pre_old = load4(p.out_tiled ? p.out + ft_index(me + p.out_row0, ne, p.ldo >> 5) : p.out + (size_t)me * p.ldo + ne);
+            if (p.gate) pre_gate = load4(p.gate + ne);
+            if (p.bias) pre_bias = load4(p.bias + ne);
+        } else if constexpr (EPI == SK_BIAS || EPI == SK_BIAS_SILU) {
+            pre_bias = load4(p.bias + ne);
+        } else if constexpr (EPI == SK_QKV_ROPE) {
+            if (ne < 2304) pre_cs = load4(p.rope + (size_t)me * 256 + (ne & 255));
+        }
+    }
     // keep every load above in flight before anything waits on one of them
     __builtin_amdgcn_sched_barrier(0);
 
@@ -160,15 +176,15 @@ void skinny_kernel(SkinnyP p) {
     bf16_t* const optr = p.out_tiled ? p.out + ft_index(m + p.out_row0, n0, p.ldo >> 5) : p.out + (size_t)m * p.ldo + n0;
     if constexpr (EPI == SK_BIAS || EPI == SK_BIAS_SILU) {
         f32x4 o = v[0];
-        const bf16x4 bb = load4(p.bias + n0);
+        const bf16x4 bb = pre_bias;
 #pragma unroll
         for (int e = 0; e < 4; ++e) { o[e] += bf2f(bb[e]); if (EPI == SK_BIAS_SILU) o[e] = siluf(o[e]); }
         store4(optr, pack4(o));
     } else if constexpr (EPI == SK_RES) {
         f32x4 o = v[0];
-        if (p.gate) { const bf16x4 gg = load4(p.gate + n0); for (int e = 0; e < 4; ++e) o[e] *= bf2f(gg[e]); }
-        if (p.bias) { const bf16x4 bb = load4(p.bias + n0); for (int e = 0; e < 4; ++e) o[e] += bf2f(bb[e]); }
-        const bf16x4 old = load4(optr);
+        if (p.gate) { for (int e = 0; e < 4; ++e) o[e] *= bf2f(pre_gate[e]); }
+        if (p.bias) { for (int e = 0; e < 4; ++e) o[e] += bf2f(pre_bias[e]); }
+        const bf16x4 old = pre_old;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] += bf2f(old[e]);
         store4(optr, pack4(o));
@@ -178,7 +194,7 @@ void skinny_kernel(SkinnyP p) {
     } else if constexpr (EPI == SK_QKV_ROPE) {
         f32x4 o = v[0];
         if (n0 < 2304) {
-            const bf16x4 cs = load4(p.rope + (size_t)m * 256 + (n0 & 255));
+            const bf16x4 cs = pre_cs;
             const float c0 = bf2f(cs[0]), s0 = bf2f(cs[1]), c1 = bf2f(cs[2]), s1 = bf2f(cs[3]);
             const f32x4 x = o;
             o[0] = x[0] * c0 - x[1] * s0; o[1] = x[1] * c0 + x[0] * s0;
