@@ -134,6 +134,7 @@ def main():
     stream = torch.cuda.current_stream().cuda_stream
     if args.traffic_probe:
         ms, name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, 4, 5, stream)
+        ctx.time_stage(capi.STAGE_SUFFIX_LAYER, -1, 0, 2, stream)          # every action-expert layer, weights cold
         src = torch.ones(COPY_PROBE_BYTES // 2, dtype=torch.bfloat16, device=dev)
         dst = torch.empty_like(src)
         for _ in range(3):
@@ -187,7 +188,10 @@ def main():
     hbm = layer_bytes / (layer_ms * 1e-3) / 1e9
     roofline_hbm = {"bound": "hbm", "kernel": "one action-expert layer (qkv, attention, o, geglu, down)",
                     "achieved": round(hbm, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hbm / HBM_PEAK_GBS, 4),
-                    "launch_ms": round(layer_ms, 4), "launch_ms_cache_warm": round(layer_warm_ms, 4), "traffic": None}
+                    "launch_ms": round(layer_ms, 4), "launch_ms_cache_warm": round(layer_warm_ms, 4),
+                    # HBM bytes per layer from rocprofv3 FETCH_SIZE + WRITE_SIZE summed over the six kernels, headline shape only
+                    # (profiles/action_expert_layer_pi0_3view_p20_c50_hbm_traffic.md)
+                    "traffic": 57.8e6 if args.config == "headline" else None, "algorithmic_bytes": layer_bytes}
     # whole-forward roofline fraction: (F_vis + F_pre) / P_mfma + B_dec / BW  over the measured p50
     v_l = 1152 * 3456 + 1152 * 1152 + 2 * 1152 * 4304
     e_l = 2048 * 2560 + 2048 * 2048 + 3 * 2048 * 16384
