@@ -14,7 +14,7 @@
 //
 // The suffix pass has only ~26 row tiles but ~840 keys, and one CU can pull only ~100 GB/s through its
 // L2 port, so a workgroup that walks all keys is bound by that port.  Its keys are therefore split over
-// gridDim.y workgroups, each writing an un-normalised partial (O, row max, row sum); a second small
+// several workgroups, each writing an un-normalised partial (O, row max, row sum); a second small
 // kernel (attn_merge_kernel) combines the partials.  Merging inside the first kernel (last workgroup to
 // finish does it) was measured slower: the partials cross XCDs, whose L2s are not coherent with each
 // other, and device-scope fences or write-through accesses cost more than one extra launch.
@@ -41,8 +41,18 @@ void mqa_kernel(AttnP p) {
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
-    const int m0 = blockIdx.x * (16 * MQ);
-    const int nsplit = gridDim.y, split = blockIdx.y;
+    // Workgroup ids are dealt round-robin over the 8 XCDs.  With a key split the id is decoded so that all row
+    // blocks of one split land on the same XCD: its slice of K / V^T is then fetched into one L2 instead of eight.
+    const int nsplit = p.nsplit_eff;
+    int rowblk, split;
+    if (nsplit == 1) { rowblk = blockIdx.x; split = 0; }
+    else {
+        const int spx = (nsplit + 7) >> 3;                           // splits per XCD
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        split = xcd + 8 * (idx % spx); rowblk = idx / spx;
+        if (split >= nsplit) return;                                 // (whole workgroup, before any barrier)
+    }
+    const int m0 = rowblk * (16 * MQ);
 
     int vl = p.prefix_alloc;
     if (p.valid_len) vl = max(0, min(*p.valid_len, p.prefix_alloc));
@@ -51,7 +61,7 @@ void mqa_kernel(AttnP p) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         // fragment-tiled Q: one contiguous 1 KB read per fragment (row tiles past the end are padding)
-        const bf16_t* qp = p.q + ((size_t)(blockIdx.x * MQ + mq) * 8 * 64 + lane) * 8;
+        const bf16_t* qp = p.q + ((size_t)(rowblk * MQ + mq) * 8 * 64 + lane) * 8;
 #pragma unroll
         for (int kd = 0; kd < 8; ++kd) qf[mq][kd] = *(const bf16x8*)(qp + kd * 512);
     }
@@ -180,7 +190,7 @@ void mqa_kernel(AttnP p) {
     }
     // partial record of one (row block, split): MQ x { O [16][64] f32x4 | max [16] | sum [16] }
     constexpr int REC = 16 * 64 * 4 + 32;
-    float* const mine = p.partial + ((size_t)blockIdx.x * nsplit + split) * (MQ * REC);
+    float* const mine = p.partial + ((size_t)rowblk * nsplit + split) * (MQ * REC);
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         __syncthreads();                       // ls written / previous obuf round consumed
@@ -349,7 +359,8 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
         if (!p.partial || nsplit > 16) return 1;
         if ((size_t)blocks * nsplit * MQ * (16 * 64 * 4 + 32) > p.partial_floats) return 3;
     }
-    hipLaunchKernelGGL(kern, dim3(blocks, nsplit), dim3(WAVES * 64), smem, s, p);
+    p.nsplit_eff = nsplit;
+    hipLaunchKernelGGL(kern, dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks), dim3(WAVES * 64), smem, s, p);
     if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
     else if (nsplit > 1) hipLaunchKernelGGL((attn_merge_kernel<MQ, 8>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
     return hipGetLastError() == hipSuccess ? 0 : 5;

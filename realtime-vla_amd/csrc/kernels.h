@@ -109,7 +109,7 @@ struct AttnP {
     int prefix_alloc; const int* valid_len; int state_rows;
     // key split over workgroups (nsplit > 1, at most 16): fp32 partial records, combined by a second launch
     int nsplit; float* partial; size_t partial_floats;
-    int kb_per_split;                // filled by the launcher
+    int kb_per_split, nsplit_eff;    // filled by the launcher
 };
 int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s);
 // SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major
