@@ -28,6 +28,25 @@ CONFIGS = {
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 COPY_PROBE_BYTES = 256 << 20   # size of the calibration copy of --traffic-probe
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def profiled_traffic(file_name, kernel_desc, workload, lib_version):
+    """HBM bytes per launch as recorded in a rocprofv3 counter summary under profiles/ (a line `facts: {json}`), or None
+    when no summary exists for exactly this kernel variant (tile and split as the library reports them), workload and
+    library version: a counter reading of an older kernel says nothing about the current one."""
+    path = os.path.join(PROFILES, file_name)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("facts:"):
+            try:
+                f = json.loads(line[len("facts:"):])
+            except ValueError:
+                return None
+            if f.get("kernel") == kernel_desc and f.get("workload") == workload and f.get("rtvla_version") == lib_version:
+                return f.get("traffic_bytes_per_launch")
+    return None
 
 
 def bench_transforms(args, dev):
@@ -98,6 +117,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    ap.add_argument("--cpu-runs", type=int, default=3, help="timed CPU-oracle forwards after one warm-up (median reported)")
     ap.add_argument("--transforms", action="store_true",
                     help="measure the observation pre-/post-processing kernels (3 camera frames of 480x640, state, actions) instead of the forward")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -132,15 +152,19 @@ def main():
         run = lambda nz: model.forward(img, nz)
     ctx = model._engine.ctx
     stream = torch.cuda.current_stream().cuda_stream
+    lib_version = capi.load().rtvla_version()
+    # index of the gate/up GEMM among the launches of one prefix layer, found by its name
+    GEGLU_LAUNCH = next(i for i in range(16) if (ctx.time_launch(capi.STAGE_PREFIX_LAYER, 0, 0, i, 1, stream) or (0, "prefix geglu"))[1].startswith("prefix geglu"))
     if args.traffic_probe:
-        ms, name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, 4, 5, stream)
+        ms, name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, GEGLU_LAUNCH, 5, stream)
         ctx.time_stage(capi.STAGE_SUFFIX_LAYER, -1, 0, 2, stream)          # every action-expert layer, weights cold
         src = torch.ones(COPY_PROBE_BYTES // 2, dtype=torch.bfloat16, device=dev)
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-        print(json.dumps({"probe": name, "launch_ms": ms, "copy_bytes": COPY_PROBE_BYTES}))
+        print(json.dumps({"probe": name, "launch_ms": ms, "copy_bytes": COPY_PROBE_BYTES, "rtvla_version": lib_version,
+                          "workload": args.config}))
         return
     # fresh noise every iteration (BASELINE config 5); drawn up front so the timed region holds only forward()
     draws = [syn.observation(seed, views, chunk, device=dev, draw=i % 16)[2] for i in range(16)]
@@ -169,16 +193,18 @@ def main():
     # dominant kernel: the Gemma-prefix GeGLU GEMM (gate and up, 2048 -> 16384 each): launch index 4 of a prefix layer
     # (cycled over the layers, so that each launch streams its 134 MB of weights from HBM as it does inside the forward;
     # repeated on one layer the weights stay in the memory-side cache and the launch is ~8 % shorter)
-    geglu_ms, geglu_name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, -1, 0, 4, 3, stream)
-    geglu_warm_ms, _ = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, 4, 20, stream)
+    geglu_ms, geglu_name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, -1, 0, GEGLU_LAUNCH, 3, stream)
+    geglu_warm_ms, _ = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, GEGLU_LAUNCH, 20, stream)
+    assert geglu_name.startswith("prefix geglu"), geglu_name
     geglu_flop = 2.0 * 2.0 * S_e * 2048 * 16384
     mfma = geglu_flop / (geglu_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": "prefix GeGLU GEMM (gemm_mfma_kernel, EPI_GEGLU), M=%d K=2048 N=2x16384" % S_e,
                 "achieved": round(mfma, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(mfma / MFMA_PEAK_TFLOPS, 4),
                 "launch_ms": round(geglu_ms, 4), "launch_ms_cache_warm": round(geglu_warm_ms, 4),
-                # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each calibrated on a 256 MiB copy; measured for
-                # the headline shape only (profiles/gemm_geglu_pi0_3view_p20_c50_hbm_traffic.md)
-                "traffic": 212.0e6 if args.config == "headline" else None,
+                # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each calibrated on a 256 MiB copy, as recorded in
+                # profiles/ for exactly this kernel variant and library version (null otherwise)
+                "traffic": profiled_traffic("gemm_geglu_hbm_traffic.md", geglu_name, args.config, lib_version),
+                "kernel_variant": geglu_name,
                 "algorithmic_bytes": 2.0 * (S_e * 2048 + 2 * 2048 * 16384 + S_e * 16384)}
     # the action-expert side: one suffix layer (5 launches) streams 18 D_L-sized weight sets per step
     layer_ms = ctx.time_stage(capi.STAGE_SUFFIX_LAYER, -1, 0, 5, stream)          # all 18 layers in turn: weights cold, as in the forward
@@ -189,9 +215,9 @@ def main():
     roofline_hbm = {"bound": "hbm", "kernel": "one action-expert layer (qkv, attention, o, geglu, down)",
                     "achieved": round(hbm, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hbm / HBM_PEAK_GBS, 4),
                     "launch_ms": round(layer_ms, 4), "launch_ms_cache_warm": round(layer_warm_ms, 4),
-                    # HBM bytes per layer from rocprofv3 FETCH_SIZE + WRITE_SIZE summed over the six kernels, headline shape only
-                    # (profiles/action_expert_layer_pi0_3view_p20_c50_hbm_traffic.md)
-                    "traffic": 57.8e6 if args.config == "headline" else None, "algorithmic_bytes": layer_bytes}
+                    # HBM bytes per layer from rocprofv3 FETCH_SIZE + WRITE_SIZE summed over the layer's kernels (profiles/)
+                    "traffic": profiled_traffic("action_expert_layer_hbm_traffic.md", "action-expert layer", args.config, lib_version),
+                    "algorithmic_bytes": layer_bytes}
     # whole-forward roofline fraction: (F_vis + F_pre) / P_mfma + B_dec / BW  over the measured p50
     v_l = 1152 * 3456 + 1152 * 1152 + 2 * 1152 * 4304
     e_l = 2048 * 2560 + 2048 * 2048 + 3 * 2048 * 16384
@@ -202,32 +228,36 @@ def main():
     ideal_ms = ((f_vis + f_pre) / (MFMA_PEAK_TFLOPS * 1e12) + b_dec / (HBM_PEAK_GBS * 1e9)) * 1e3
 
     result = {
-        "metric": "p50 ms per Pi0 forward (3 views, chunk 50, 10 steps); % roofline",
+        "metric": "p50 ms per %s forward (%d views, chunk %d, 10 steps); %% roofline" % ("Pi0" if model_name == "pi0" else "Pi05", views, chunk),
         "value": round(p50, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(t_all / args.steps, 4), "p99_ms": round(p99, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": desc, "config_id": args.config, "S_v": S_v, "S_e": S_e, "S_d": S_d, "keys": keys,
-                   "graph_launches": model._engine.graph_launches, "weights": "seeded N(0, 0.02^2) bf16, norms = 1"},
+                   "graph_launches": model._engine.graph_launches, "weights": "seeded N(0, 0.02^2) bf16, norms = 1",
+                   "rtvla_version": lib_version},
         "roofline": roofline, "roofline_hbm": roofline_hbm,
         "forward_roofline_frac": round(ideal_ms / p50, 4), "forward_ideal_ms": round(ideal_ms, 4),
         "reference_published": {"value_ms": 39.2, "hardware": "RTX 4090, Triton", "source": "README.md:18"} if args.config == "headline" else None,
     }
 
-    # ---- CPU baseline: the oracle (a port of the reference math) on the host cores, one forward ----
+    # ---- CPU baseline: the oracle (a port of the reference math) on the host cores: 1 warm-up + 3 timed forwards, median ----
     if not args.no_cpu:
         from oracle import pi0 as o0, pi05 as o5          # the checker, timed as a baseline only
         cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or os.cpu_count()
         torch.set_num_threads(cores)
         ckc = {k: v.cpu() for k, v in ck.items()}
-        t0 = time.perf_counter()
-        if model_name == "pi0":
-            ref = o0.forward(ckc, img.cpu(), state.cpu(), draws[0].cpu())
-        else:
-            ref = o5.forward(ckc, img.cpu(), draws[0].cpu())
-        cpu_ms = (time.perf_counter() - t0) * 1e3
+        imgc, statec, noisec = img.cpu(), state.cpu(), draws[0].cpu()
+        cpu_times = []
+        for it in range(1 + args.cpu_runs):
+            t0 = time.perf_counter()
+            ref = o0.forward(ckc, imgc, statec, noisec) if model_name == "pi0" else o5.forward(ckc, imgc, noisec)
+            if it:
+                cpu_times.append((time.perf_counter() - t0) * 1e3)
+        cpu_ms = sorted(cpu_times)[len(cpu_times) // 2]
         out = run(draws[0]).float().cpu()
         result["cpu_baseline"] = {"value": round(cpu_ms, 1), "unit": "ms", "cores": cores, "kind": "port",
-                                  "sample": "one forward of the same workload (no warm-up), PyTorch CPU eager oracle"}
+                                  "sample": "median of %d forwards of the same workload after 1 warm-up, PyTorch CPU eager oracle" % args.cpu_runs,
+                                  "runs_ms": [round(t, 1) for t in cpu_times]}
         result["action_mae_vs_oracle"] = round((out - ref).abs().mean().item(), 5)
     print(json.dumps(result))
 

@@ -66,7 +66,9 @@ enum rtvla_stage {
     RTVLA_STAGE_SUFFIX_STEP_END = 7 /* pi0_infer.py:1224-1230 / pi05_infer.py:511-523 Euler update   */
 };
 
-/* Library build / ABI version (no reference counterpart). */
+/* Library version (no reference counterpart): raised whenever a kernel or the schedule changes, so that a
+ * measurement recorded for one version is not mistaken for the current kernels. */
+#define RTVLA_VERSION 2
 int rtvla_version(void);
 
 /* Create a context for one shape set.  Replaces the tensor allocation block of
@@ -134,6 +136,8 @@ int rtvla_forward_stage(rtvla_ctx* ctx, int stage, int layer, int step, void* hi
 /* Capture rtvla_forward into a HIP graph held by the context / replay it on a stream.
  * Replaces record_infer_graph and infer_graph.replay() (pi0_infer.py:1347-1354, :1360). */
 int rtvla_graph_capture(rtvla_ctx* ctx, void* hip_stream);
+/* A graph records the addresses bound at capture time: rtvla_bind and rtvla_bind_workspace drop it, and
+ * rtvla_graph_launch then returns RTVLA_ERR_STATE until rtvla_prepare and rtvla_graph_capture have run again. */
 int rtvla_graph_launch(rtvla_ctx* ctx, void* hip_stream);
 
 /* Number of kernels the last forward (or stage) enqueued: the kernel nodes of the captured graph. */
@@ -158,11 +162,28 @@ int rtvla_time_launch(rtvla_ctx* ctx, int stage, int layer, int step, int launch
  * individually with HIP events on the stream; writes per-iteration milliseconds to ms_out[iters]. */
 int rtvla_time_forward(rtvla_ctx* ctx, int iters, void* hip_stream, float* ms_out);
 
-/* Unit-level entry points used by the parity tests: run one kernel family on caller tensors.
- * `w_tiled` comes from rtvla_pretile.  (No reference counterpart; the reference's per-kernel
- * wrappers, e.g. pi0_infer.py:396-419, :727-733, take torch tensors.) */
+/* Unit-level entry points used by the per-kernel parity tests: one kernel family on caller tensors.  (No reference
+ * counterpart as an ABI; they stand where the reference's per-shape wrappers stand, e.g. matmul_small_bias
+ * pi0_infer.py:126-158, matmul_split_k + merge_split_k_bias_res :292-346, matmul_k_1024_1024_bias :927-937.)
+ *
+ * rtvla_pretile: W[K][N] bf16 row-major -> the 16-column x 32-row MFMA fragment order the action-expert kernels
+ * stream (rtvla_pretile_elems elements).
+ *
+ * rtvla_linear: out[M][N] = x[M][K] w[K][N] + bias[N] (bias may be null), all bf16 row-major, fp32 accumulation,
+ * K a multiple of 8, N a multiple of 16.  `tile` selects the kernel: 0 .. count-1 one block tile of the large-M MFMA
+ * GEMM (rtvla_linear_tile_shape tells its rows x columns and fails past the last one), -1 the tile the forward's
+ * cost model picks for this shape, RTVLA_TILE_SKINNY the weight-streaming kernel of the action expert (M <= 64,
+ * K = 1024, 2048 or 4096).  `nsplit`: 1 = one pass with the bias epilogue; 2..8 = split-K into fp32 partials that the
+ * reduce kernel sums (N <= 2048); 0 = the split the cost model picks, through the partial + reduce route the
+ * residual GEMMs of the forward take.  RTVLA_ERR_LIMIT when the tile cannot take the shape (the tiles of more than
+ * 128 rows consume K in steps of 128 per split).  `workspace`: rtvla_linear_workspace_bytes, 256-byte aligned. */
+#define RTVLA_TILE_SKINNY (-2)
 size_t rtvla_pretile_elems(int K, int N);
 int rtvla_pretile(const void* w, int K, int N, void* w_tiled, void* hip_stream);
+size_t rtvla_linear_workspace_bytes(int M, int K, int N, int tile, int nsplit);
+int rtvla_linear(const void* x, int M, int K, const void* w, int N, const void* bias, void* out, void* workspace,
+                 size_t workspace_bytes, int tile, int nsplit, void* hip_stream);
+int rtvla_linear_tile_shape(int tile, int* rows, int* cols);
 
 /* ---- observation pre-/post-processing either side of the forward (context-free, capturable) ----------------
  * The reference does these on the host per observation (test.py:88-201).  All pointers are device pointers. */

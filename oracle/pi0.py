@@ -9,6 +9,18 @@ from . import ops
 from .ops import f32, gemm
 
 
+def vision_layer(w, i, x, rnd):
+    """pi0_infer.py:607-646, one SigLIP layer: LN -> QKV(+bias) -> attention -> O(+bias) + residual ->
+    LN -> up(+bias) -> GELU -> down(+bias) + residual."""
+    n = rnd(ops.layer_norm(x, w["vision_pre_attn_norm_w"][i], w["vision_pre_attn_norm_b"][i]))
+    qkv = rnd(f32(w["vision_attn_qkv_b"][i]) + gemm(n, w["vision_attn_qkv_w"][i]))
+    a = ops.vision_attention(qkv, rnd)
+    x = rnd(x + f32(w["vision_attn_o_b"][i]) + gemm(a, w["vision_attn_o_w"][i]))
+    n = rnd(ops.layer_norm(x, w["vision_pre_ffn_norm_w"][i], w["vision_pre_ffn_norm_b"][i]))
+    h = rnd(ops.gelu_tanh(f32(w["vision_ffn_up_b"][i]) + gemm(n, w["vision_ffn_up_w"][i])))
+    return rnd(x + f32(w["vision_ffn_down_b"][i]) + gemm(h, w["vision_ffn_down_w"][i]))
+
+
 def vision_encoder(w, images, rnd, taps=None):
     """pi0_infer.py:598-646 -> vision_x [v*256, 1152]."""
     x = ops.patches(f32(images))
@@ -17,13 +29,7 @@ def vision_encoder(w, images, rnd, taps=None):
     if taps is not None:
         taps["vision_embed"] = x.clone()
     for i in range(w["vision_attn_qkv_w"].shape[0]):
-        n = rnd(ops.layer_norm(x, w["vision_pre_attn_norm_w"][i], w["vision_pre_attn_norm_b"][i]))
-        qkv = rnd(f32(w["vision_attn_qkv_b"][i]) + gemm(n, w["vision_attn_qkv_w"][i]))
-        a = ops.vision_attention(qkv, rnd)
-        x = rnd(x + f32(w["vision_attn_o_b"][i]) + gemm(a, w["vision_attn_o_w"][i]))
-        n = rnd(ops.layer_norm(x, w["vision_pre_ffn_norm_w"][i], w["vision_pre_ffn_norm_b"][i]))
-        h = rnd(ops.gelu_tanh(f32(w["vision_ffn_up_b"][i]) + gemm(n, w["vision_ffn_up_w"][i])))
-        x = rnd(x + f32(w["vision_ffn_down_b"][i]) + gemm(h, w["vision_ffn_down_w"][i]))
+        x = vision_layer(w, i, x, rnd)
         if taps is not None:
             taps["vision_x/%d" % i] = x.clone()
     return x
@@ -79,6 +85,36 @@ def transformer_encoder(w, x, rnd, taps=None, valid_len=None):
     return ks, vs
 
 
+def suffix_layer(w, i, x, k_prefix, v_prefix, table, mask, rnd):
+    """pi0_infer.py:1186-1223, one action-expert layer over the suffix rows x [S_d, 1024] (row 0 = state token):
+    RMS factor -> QKV (factor applied to the fp32 accumulator, :1005) -> RoPE -> K/V appended behind the prefix
+    rows of this layer's cache (:1191-1192) -> masked attention (:1085) -> O + residual -> RMS factor ->
+    GeGLU on the pre-scaled rows (:718) -> down + residual."""
+    s_d = x.shape[0]
+    f = rnd(ops.rms_factor(x))
+    acc = gemm(x, w["decoder_attn_qkv_w"][i]) * f
+    q = rnd(ops.rope_interleaved(acc[:, :2048], table))
+    k = rnd(ops.rope_interleaved(acc[:, 2048:2304], table))
+    v = rnd(acc[:, 2304:])
+    kk = torch.cat([k_prefix, k], dim=0)
+    vv = torch.cat([v_prefix, v], dim=0)
+    a = ops.mqa_attention(q.reshape(-1, 256), kk, vv, rnd, mask).reshape(s_d, 2048)
+    x = rnd(x + gemm(a, w["decoder_attn_o_w"][i]))
+    f = rnd(ops.rms_factor(x))
+    xs = rnd(x * f)                                               # bf16 x * bf16 f -> bf16 before the dot (:718)
+    g = rnd(ops.gelu_tanh(gemm(xs, w["decoder_ffn_gate_w"][i])) * gemm(xs, w["decoder_ffn_up_w"][i]))
+    return rnd(x + gemm(g, w["decoder_ffn_down_w"][i]))
+
+
+def euler_step(w, x, noise, rnd):
+    """pi0_infer.py:953-964, :1224-1230: noise += (x[1:] * f) W_out + b_out (dt and the final norm scale are
+    folded into W_out, b_out by the converter)."""
+    xo = x[1:]
+    f = rnd(ops.rms_factor(xo))
+    xs = rnd(xo * f)                                              # :113
+    return rnd(noise + f32(w["decoder_action_fused_out_proj_b"]) + gemm(xs, w["decoder_action_fused_out_proj_w"]))
+
+
 def transformer_decoder(w, ks, vs, state, noise, rnd, taps=None, num_steps=10):
     """pi0_infer.py:1165-1230: state token + 10 Euler flow steps over the action expert."""
     s_e = ks[0].shape[0]
@@ -96,25 +132,10 @@ def transformer_decoder(w, ks, vs, state, noise, rnd, taps=None, num_steps=10):
         if taps is not None:
             taps["decoder_in/%d" % t] = x.clone()
         for i in range(layers):
-            f = rnd(ops.rms_factor(x))
-            acc = gemm(x, w["decoder_attn_qkv_w"][i]) * f            # scale applied to the fp32 accumulator (:1005)
-            q = rnd(ops.rope_interleaved(acc[:, :2048], table))
-            k = rnd(ops.rope_interleaved(acc[:, 2048:2304], table))
-            v = rnd(acc[:, 2304:])
-            kk = torch.cat([ks[i], k], dim=0)
-            vv = torch.cat([vs[i], v], dim=0)
-            a = ops.mqa_attention(q.reshape(-1, 256), kk, vv, rnd, mask).reshape(s_d, 2048)
-            x = rnd(x + gemm(a, w["decoder_attn_o_w"][i]))
-            f = rnd(ops.rms_factor(x))
-            xs = rnd(x * f)                                           # bf16 x * bf16 f -> bf16 before the dot (:718)
-            g = rnd(ops.gelu_tanh(gemm(xs, w["decoder_ffn_gate_w"][i])) * gemm(xs, w["decoder_ffn_up_w"][i]))
-            x = rnd(x + gemm(g, w["decoder_ffn_down_w"][i]))
+            x = suffix_layer(w, i, x, ks[i], vs[i], table, mask, rnd)
             if taps is not None:
                 taps["decoder_x/%d/%d" % (t, i)] = x.clone()
-        xo = x[1:]
-        f = rnd(ops.rms_factor(xo))
-        xs = rnd(xo * f)                                              # :113
-        noise = rnd(noise + f32(w["decoder_action_fused_out_proj_b"]) + gemm(xs, w["decoder_action_fused_out_proj_w"]))
+        noise = euler_step(w, x, noise, rnd)
         if taps is not None:
             taps["noise/%d" % t] = noise.clone()
     return noise

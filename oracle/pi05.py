@@ -34,6 +34,25 @@ def adarms(x, style, rnd):
     return rnd(x * ops.rms_factor(x) * (1.0 + scale) + shift), gate
 
 
+def suffix_layer(w, i, x, k_prefix, v_prefix, style_attn, style_ffn, table, mask, rnd):
+    """pi05_infer.py:427-509, one action-expert layer: adaRMS(attention style) -> QKV -> RoPE -> K/V appended
+    behind the allocated prefix rows -> prefix/suffix-masked attention -> gated O + residual ->
+    adaRMS(FFN style) -> GeGLU -> gated down + residual."""
+    s_d = x.shape[0]
+    n, gate = adarms(x, style_attn, rnd)
+    acc = gemm(n, w["decoder_attn_qkv_w"][i])
+    q = rnd(ops.rope_interleaved(acc[:, :2048], table))
+    k = rnd(ops.rope_interleaved(acc[:, 2048:2304], table))
+    v = rnd(acc[:, 2304:])
+    kk = torch.cat([k_prefix, k], dim=0)
+    vv = torch.cat([v_prefix, v], dim=0)
+    a = ops.mqa_attention(q.reshape(-1, 256), kk, vv, rnd, mask).reshape(s_d, 2048)
+    x = rnd(x + gemm(a, w["decoder_attn_o_w"][i]) * gate)         # pi05_infer.py:58
+    n, gate = adarms(x, style_ffn, rnd)
+    g = rnd(ops.gelu_tanh(gemm(n, w["decoder_ffn_gate_w"][i])) * gemm(n, w["decoder_ffn_up_w"][i]))
+    return rnd(x + gemm(g, w["decoder_ffn_down_w"][i]) * gate)
+
+
 def transformer_decoder(w, ks, vs, noise, valid_len, rnd, taps=None, num_steps=10):
     """pi05_infer.py:418-523.  `ks`/`vs` hold the allocated prefix rows (valid or not); suffix
     RoPE positions start at valid_len - 1 (pi05_infer.py:787-790)."""
@@ -49,18 +68,7 @@ def transformer_decoder(w, ks, vs, noise, valid_len, rnd, taps=None, num_steps=1
         if taps is not None:
             taps["decoder_in/%d" % t] = x.clone()
         for i in range(layers):
-            n, gate = adarms(x, st_attn[t][i], rnd)
-            acc = gemm(n, w["decoder_attn_qkv_w"][i])
-            q = rnd(ops.rope_interleaved(acc[:, :2048], table))
-            k = rnd(ops.rope_interleaved(acc[:, 2048:2304], table))
-            v = rnd(acc[:, 2304:])
-            kk = torch.cat([ks[i], k], dim=0)
-            vv = torch.cat([vs[i], v], dim=0)
-            a = ops.mqa_attention(q.reshape(-1, 256), kk, vv, rnd, mask).reshape(s_d, 2048)
-            x = rnd(x + gemm(a, w["decoder_attn_o_w"][i]) * gate)     # pi05_infer.py:58
-            n, gate = adarms(x, st_ffn[t][i], rnd)
-            g = rnd(ops.gelu_tanh(gemm(n, w["decoder_ffn_gate_w"][i])) * gemm(n, w["decoder_ffn_up_w"][i]))
-            x = rnd(x + gemm(g, w["decoder_ffn_down_w"][i]) * gate)
+            x = suffix_layer(w, i, x, ks[i], vs[i], st_attn[t][i], st_ffn[t][i], table, mask, rnd)
             if taps is not None:
                 taps["decoder_x/%d/%d" % (t, i)] = x.clone()
         n, _ = adarms(x, st_final[t], rnd)

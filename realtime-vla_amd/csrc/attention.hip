@@ -368,14 +368,11 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
 
 }  // namespace
 
-int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s) {
+int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s) {
     if (p.rows <= 0 || p.keys <= 0 || (p.ldvt & 63) || p.ldvt < ((p.keys + 63) / 64) * 64) return 1;
-    switch (waves) {                                            // variant: waves, row tiles and 16-key tiles per wave round
-        case 4: return launch_mqa_inst<4, 2, 2>(p, s);          // prefix pass
-        case 8: return launch_mqa_inst<4, 1, 4>(p, s);          // suffix pass: few rows, one row tile per workgroup
-        case 9: return launch_mqa_inst<2, 1, 4>(p, s);
-        case 10: return launch_mqa_inst<4, 1, 2>(p, s);
-        case 11: return launch_mqa_inst<2, 2, 2>(p, s);
+    switch (variant) {                                          // template: waves, row tiles per workgroup, 16-key tiles per wave round
+        case ATTN_PREFIX: return launch_mqa_inst<4, 2, 2>(p, s);
+        case ATTN_SUFFIX: return launch_mqa_inst<4, 1, 2>(p, s);
     }
     return 2;
 }

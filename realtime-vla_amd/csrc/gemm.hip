@@ -356,11 +356,9 @@ int launch_cfg(const GemmP& p, hipStream_t s) {
 template <int EPI>
 int launch_epi(const GemmP& p, int tile, hipStream_t s) {
     switch (tile) {
-        case TILE_256x256: return launch_cfg<4, 8, 2, EPI>(p, s);
         case TILE_224x256: return launch_cfg<4, 7, 2, EPI>(p, s);
         case TILE_160x256: return launch_cfg<4, 5, 2, EPI>(p, s);
         case TILE_128x256: return launch_cfg<4, 4, 2, EPI>(p, s);
-        case TILE_96x256:  return launch_cfg<4, 3, 2, EPI>(p, s);
         case TILE_64x256:  return launch_cfg<4, 2, 2, EPI>(p, s);
         case TILE_64x128:  if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 2, 1, EPI>(p, s); else return 2;
         case TILE_128x128: if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 4, 1, EPI>(p, s); else return 2;
@@ -370,7 +368,7 @@ int launch_epi(const GemmP& p, int tile, hipStream_t s) {
 
 }  // namespace
 
-int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {256, 224, 160, 128, 96, 64, 64, 128}; return v[tile]; }
+int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {224, 160, 128, 64, 64, 128}; return v[tile]; }
 int gemm_tile_bn(int tile) { return tile >= TILE_64x128 ? 128 : 256; }
 
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {

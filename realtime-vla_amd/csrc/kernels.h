@@ -49,7 +49,7 @@ struct GemmP {
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt;
 };
 // workgroup tile (rows x columns), 4 waves each owning 64 columns (two 32-column MFMA tiles)
-enum GemmTile { TILE_256x256 = 0, TILE_224x256, TILE_160x256, TILE_128x256, TILE_96x256, TILE_64x256, TILE_64x128, TILE_128x128, TILE_COUNT };
+enum GemmTile { TILE_224x256 = 0, TILE_160x256, TILE_128x256, TILE_64x256, TILE_64x128, TILE_128x128, TILE_COUNT };
 int gemm_tile_bm(int tile);
 int gemm_tile_bn(int tile);
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s);
@@ -111,7 +111,8 @@ struct AttnP {
     int nsplit; float* partial; size_t partial_floats;
     int kb_per_split, nsplit_eff;    // filled by the launcher
 };
-int launch_mqa_attention(const AttnP& p, int waves, hipStream_t s);
+enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1 };    // many rows, two row tiles per workgroup / few rows, one row tile and a key split
+int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s);
 // SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major
 void launch_vision_attention(const bf16_t* q, const bf16_t* k, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);
 

@@ -86,9 +86,7 @@ struct rtvla_ctx {
     }
     bf16_t* TW(const char* n, int layer = 0) { const WsBuf& b = BI(n); return (bf16_t*)(ws + b.offset) + (size_t)b.ld * layer; }
 
-    // suffix attention: kernel variant and key split (RTVLA_ATTN_VARIANT / RTVLA_ATTN_SPLIT override, for tuning)
-    int attn_variant = getenv("RTVLA_ATTN_VARIANT") ? atoi(getenv("RTVLA_ATTN_VARIANT")) : 10;
-    int attn_split = getenv("RTVLA_ATTN_SPLIT") ? atoi(getenv("RTVLA_ATTN_SPLIT")) : 0;      // 0: one workgroup per 128 keys
+    int attn_split = 0;            // suffix attention key split; 0: one workgroup per 128 keys
 
     int only = -1;                 // >= 0: enqueue only the launch with this index (per-kernel timing)
     std::string last_name;
@@ -119,14 +117,17 @@ constexpr int64_t ATTN_PARTIAL_FLOATS = 32 * 16 * (16 * 64 * 4 + 32);   // 32 ro
 // their load latency; all workgroups together cannot pull more than ~20 TB/s out of L2; every launch pays a
 // fixed ramp and an epilogue that grows with the tile; split-K adds the reduce pass over the fp32 partials.
 TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what) {
-    static const int tiles[] = {TILE_224x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};   // 96x256 never won a sweep
+    static const int tiles[] = {TILE_224x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};
     static const int splits[] = {1, 2, 3, 4, 6, 8};
-    const char* only_for = getenv("RTVLA_FORCE_FOR");          // tuning aid: force tile / split for launches whose name contains this
+#ifdef RTVLA_TUNING
+    // tuning builds only: force tile / split for the launches whose name contains RTVLA_FORCE_FOR
+    const char* only_for = getenv("RTVLA_FORCE_FOR");
     if (const char* e = (only_for && !strstr(what, only_for)) ? nullptr : getenv("RTVLA_FORCE_TILE")) {
         TileChoice c{atoi(e), 1};
         if (const char* s = getenv("RTVLA_FORCE_SPLIT")) if (splittable) c.nsplit = atoi(s);
         return c;
     }
+#endif
     double best = 1e30; TileChoice bc{TILE_128x256, 1};
     for (int tile : tiles) {
         const int bm = gemm_tile_bm(tile);
@@ -156,8 +157,10 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
             if (t < best) { best = t; bc = TileChoice{tile, sp}; }
         }
     }
+#ifdef RTVLA_TUNING
     if (getenv("RTVLA_PRINT_TILES")) fprintf(stderr, "rtvla tile choice: %-18s M=%d N=%d stages=%d -> %dx%d split %d (model %.1f us)\n", what, M, ncols16 * 16,
                                              stages, gemm_tile_bm(bc.tile), gemm_tile_bn(bc.tile), bc.nsplit, best);
+#endif
     return bc;
 }
 
@@ -323,7 +326,12 @@ struct Sched {
             p.partial = c->B<float>("splitk_partial"); p.ldp = N; p.pstride = (size_t)M * N;
         }
         last_split = tc.nsplit;
-        if (c->want(what)) c->note(launch_gemm(p, epi, tc.tile, s), what);
+        if (c->want(what)) {
+            // the name a measurement reports carries the kernel variant: block tile and split-K factor
+            c->last_name = std::string(what) + " [" + std::to_string(gemm_tile_bm(tc.tile)) + "x" + std::to_string(gemm_tile_bn(tc.tile)) +
+                           " split " + std::to_string(tc.nsplit) + "]";
+            c->note(launch_gemm(p, epi, tc.tile, s), what);
+        }
     }
     int last_split = 1;
 
@@ -395,7 +403,7 @@ struct Sched {
         a.q = c->B("encoder_Q"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
         a.out = c->B("encoder_attn"); a.ldo = 256; a.out_tiled = 0; a.rows = 8 * S_e; a.keys = S_e; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = 0;
-        if (c->want("prefix attn")) c->note(launch_mqa_attention(a, 4, s), "prefix attn");
+        if (c->want("prefix attn")) c->note(launch_mqa_attention(a, ATTN_PREFIX, s), "prefix attn");
         gemm(c->B("encoder_attn"), 2048, S_e, S_e, c->TW("t_encoder_attn_o_w", i), nullptr, 2048, 2048, EPI_PARTIAL, GemmP{}, "prefix o");
         reduce(S_e, 2048, nullptr, c->B("encoder_x"), 2048, c->B("encoder_x"), 2048, c->B("encoder_x_norm"), XN_LD, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix o reduce");
         GemmP g{}; g.out = c->B("encoder_hidden"); g.ldo = EHID_LD;
@@ -455,7 +463,7 @@ struct Sched {
         a.out = c->B("decoder_attn"); a.ldo = 256; a.out_tiled = 1; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
         a.nsplit = c->attn_split > 0 ? c->attn_split : std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
-        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, c->attn_variant, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
+        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_SUFFIX, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
         skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
         SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 4096;
@@ -578,11 +586,17 @@ int hip_fail(rtvla_ctx* c, hipError_t e, const char* what) {
     return c->fail(RTVLA_ERR_DEVICE, std::string(what) + ": " + hipGetErrorString(e));
 }
 
+// A captured graph holds the addresses that were bound when it was recorded: any later binding makes it stale.
+void drop_graph(rtvla_ctx* c) {
+    if (c->exec) { hipGraphExecDestroy(c->exec); c->exec = nullptr; }
+    if (c->graph) { hipGraphDestroy(c->graph); c->graph = nullptr; }
+}
+
 }  // namespace
 
 extern "C" {
 
-int rtvla_version(void) { return 1; }
+int rtvla_version(void) { return RTVLA_VERSION; }
 
 int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out) {
     if (!dims || !out) return RTVLA_ERR_ARG;
@@ -610,8 +624,7 @@ int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out) {
 
 int rtvla_destroy(rtvla_ctx* c) {
     if (!c) return RTVLA_ERR_ARG;
-    if (c->exec) hipGraphExecDestroy(c->exec);
-    if (c->graph) hipGraphDestroy(c->graph);
+    drop_graph(c);
     delete c;
     return RTVLA_OK;
 }
@@ -644,6 +657,7 @@ int rtvla_bind(rtvla_ctx* c, const char* name, void* ptr, size_t bytes) {
     if (((uintptr_t)ptr & 15) != 0) return c->fail(RTVLA_ERR_ARG, std::string("pointer not 16-byte aligned: ") + name);
     t.ptr = ptr; t.bound = true;
     c->prepared = false;
+    drop_graph(c);
     return RTVLA_OK;
 }
 
@@ -654,6 +668,7 @@ int rtvla_bind_workspace(rtvla_ctx* c, void* ptr, size_t bytes) {
     if (bytes < c->ws_bytes) return c->fail(RTVLA_ERR_SIZE, "workspace too small");
     if (((uintptr_t)ptr & 255) != 0) return c->fail(RTVLA_ERR_ARG, "workspace not 256-byte aligned");
     c->ws = (char*)ptr; c->prepared = false;
+    drop_graph(c);
     return RTVLA_OK;
 }
 
@@ -705,8 +720,7 @@ int rtvla_graph_capture(rtvla_ctx* c, void* stream) {
     if (int rc = rtvla_forward(c, stream)) return rc;
     hipError_t e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(c, e, "eager forward before capture");
-    if (c->exec) { hipGraphExecDestroy(c->exec); c->exec = nullptr; }
-    if (c->graph) { hipGraphDestroy(c->graph); c->graph = nullptr; }
+    drop_graph(c);
     e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) return hip_fail(c, e, "hipStreamBeginCapture");
     c->status = 0; c->launches = 0; c->kernels = 0;
@@ -721,7 +735,7 @@ int rtvla_graph_capture(rtvla_ctx* c, void* stream) {
 
 int rtvla_graph_launch(rtvla_ctx* c, void* stream) {
     if (!c) return RTVLA_ERR_ARG;
-    if (!c->exec) return c->fail(RTVLA_ERR_STATE, "no graph captured");
+    if (!c->exec || !c->prepared) return c->fail(RTVLA_ERR_STATE, "no graph captured since the last rtvla_bind / rtvla_prepare");
     hipError_t e = hipGraphLaunch(c->exec, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(c, e, "hipGraphLaunch");
     return RTVLA_OK;
@@ -805,7 +819,7 @@ int rtvla_time_forward(rtvla_ctx* c, int iters, void* stream, float* ms_out) {
     int rc = 0;
     for (int i = 0; i < iters && !rc; ++i) {
         hipEventRecord(a, s);
-        rc = c->exec ? rtvla_graph_launch(c, stream) : rtvla_forward(c, stream);
+        rc = c->exec ? rtvla_graph_launch(c, stream) : rtvla_forward(c, stream);      // (a re-bind drops the graph)
         hipEventRecord(b, s);
         hipError_t e = hipEventSynchronize(b);
         if (e != hipSuccess) rc = hip_fail(c, e, "time_forward");
@@ -813,6 +827,103 @@ int rtvla_time_forward(rtvla_ctx* c, int iters, void* stream, float* ms_out) {
     }
     hipEventDestroy(a); hipEventDestroy(b);
     return rc;
+}
+
+// ---- unit-level linear layer on caller tensors (per-kernel parity tests) ----
+namespace {
+struct LinearPlan { size_t a_off, w_off, bias_off, part_off, total; int K128, tile, nsplit; bool skinny, partial; };
+
+int plan_linear(int M, int K, int N, int tile, int nsplit, LinearPlan* pl) {
+    if (M <= 0 || K <= 0 || N <= 0 || (K & 7) || (N & 15) || nsplit < 0 || nsplit > 8) return RTVLA_ERR_ARG;
+    LinearPlan p{};
+    p.skinny = tile == RTVLA_TILE_SKINNY;
+    p.K128 = k32_padded(K) * 32;
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    if (p.skinny) {
+        if (M > 64 || (K != 1024 && K != 2048 && K != 4096) || nsplit > 1) return RTVLA_ERR_LIMIT;
+        p.tile = tile; p.nsplit = 1;
+        p.w_off = 0; p.bias_off = up(tiled_elems(K, N) * 2); p.total = p.bias_off + up((size_t)N * 2);
+        *pl = p; return RTVLA_OK;
+    }
+    if (tile >= (int)TILE_COUNT || tile < -1) return RTVLA_ERR_ARG;
+    TileChoice tc{tile, nsplit < 1 ? 1 : nsplit};
+    if (tile < 0) {
+        tc = choose_tile(M, n16_tiles(N), k32_padded(K) / 2, false, nsplit == 0, "linear");
+        if (nsplit >= 1) tc.nsplit = nsplit;
+    }
+    p.tile = tc.tile; p.nsplit = tc.nsplit;
+    p.partial = nsplit == 0 || tc.nsplit > 1;              // the residual-GEMM route: fp32 partials + reduce
+    if (p.partial && N > 2048) return RTVLA_ERR_LIMIT;     // the reduce kernel handles rows of at most 2048 columns
+    p.a_off = 0;
+    p.w_off = up((size_t)M * p.K128 * 2);
+    p.bias_off = p.w_off + up(tiled_elems_wide(K, N, 8) * 2);
+    p.part_off = p.bias_off + up((size_t)N * 2);
+    p.total = p.part_off + (p.partial ? up((size_t)p.nsplit * M * N * 4) : 0);
+    *pl = p; return RTVLA_OK;
+}
+}  // namespace
+
+size_t rtvla_linear_workspace_bytes(int M, int K, int N, int tile, int nsplit) {
+    LinearPlan pl;
+    return plan_linear(M, K, N, tile, nsplit, &pl) == RTVLA_OK ? pl.total : 0;
+}
+
+int rtvla_linear(const void* x, int M, int K, const void* w, int N, const void* bias, void* out, void* workspace, size_t workspace_bytes,
+                 int tile, int nsplit, void* stream) {
+    if (!x || !w || !out || !workspace || ((uintptr_t)workspace & 255)) return RTVLA_ERR_ARG;
+    LinearPlan pl;
+    if (int rc = plan_linear(M, K, N, tile, nsplit, &pl)) return rc;
+    if (workspace_bytes < pl.total) return RTVLA_ERR_SIZE;
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    bf16_t* zbias = (bf16_t*)(ws + pl.bias_off);
+    launch_fill_zero(zbias, ((size_t)N * 2 + 255) & ~(size_t)255, s);
+    const bf16_t* b = bias ? (const bf16_t*)bias : zbias;
+    int rc = 0;
+    if (pl.skinny) {
+        bf16_t* wt = (bf16_t*)(ws + pl.w_off);
+        launch_pretile((const bf16_t*)w, K, N, wt, 1, 0, s);
+        SkinnyP p{};
+        p.A = (const bf16_t*)x; p.lda = K; p.M = M; p.B0 = wt; p.K = K; p.N16 = n16_tiles(N); p.K32p = k32_padded(K);
+        p.norm = SN_NONE; p.eps = 1e-6f; p.out = (bf16_t*)out; p.ldo = N; p.bias = b;
+        if (K == 1024) rc = launch_skinny(p, SK_BIAS, s);
+        else {
+            // the K = 2048 / 4096 variants exist with the residual epilogue only (O and down projections): out = 0 + acc + bias
+            launch_fill_zero(out, (size_t)M * N * 2, s);
+            rc = launch_skinny(p, SK_RES, s);
+        }
+    } else {
+        bf16_t* a = (bf16_t*)(ws + pl.a_off);
+        bf16_t* wt = (bf16_t*)(ws + pl.w_off);
+        launch_fill_zero(a, ((size_t)M * pl.K128 * 2 + 255) & ~(size_t)255, s);       // K is zero-padded to the 128-wide stage pair
+        launch_copy_rows((const bf16_t*)x, K, a, pl.K128, M, K, s);
+        launch_pretile((const bf16_t*)w, K, N, wt, 8, 1, s);
+        GemmP p{};
+        p.A = a; p.lda = pl.K128; p.a_rows = M; p.M = M; p.B0 = wt; p.bgroup = 8;
+        p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.nsplit = pl.nsplit;
+        if (pl.partial) {
+            float* part = (float*)(ws + pl.part_off);
+            p.partial = part; p.ldp = N; p.pstride = (size_t)M * N;
+            rc = launch_gemm(p, EPI_PARTIAL, pl.tile, s);
+            if (!rc) {
+                ReduceP r{};
+                r.partial = part; r.pstride = p.pstride; r.ldp = N; r.nsplit = pl.nsplit; r.bias = b;
+                r.x = (bf16_t*)out; r.ldx = N; r.M = M; r.N = N; r.norm = NORM_NONE;
+                rc = launch_reduce(r, s);
+            }
+        } else {
+            p.out = (bf16_t*)out; p.ldo = N; p.bias = b;
+            rc = launch_gemm(p, EPI_BIAS, pl.tile, s);
+        }
+    }
+    if (rc) return rc == 3 ? RTVLA_ERR_LIMIT : RTVLA_ERR_DEVICE;      // 3: this tile cannot take this K / split
+    return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
+}
+
+int rtvla_linear_tile_shape(int tile, int* rows, int* cols) {
+    if (tile < 0 || tile >= (int)TILE_COUNT || !rows || !cols) return RTVLA_ERR_ARG;
+    *rows = gemm_tile_bm(tile); *cols = gemm_tile_bn(tile);
+    return RTVLA_OK;
 }
 
 size_t rtvla_pretile_elems(int K, int N) { return (K > 0 && N > 0) ? tiled_elems(K, N) : 0; }

@@ -20,7 +20,8 @@ STAGE_SUFFIX_STEP_BEGIN = 5
 STAGE_SUFFIX_LAYER = 6
 STAGE_SUFFIX_STEP_END = 7
 
-ERR_NAME, ERR_SIZE = 2, 3
+ERR_NAME, ERR_SIZE, ERR_STATE, ERR_LIMIT = 2, 3, 4, 7
+TILE_AUTO, TILE_SKINNY = -1, -2
 
 
 class Dims(ctypes.Structure):
@@ -59,6 +60,9 @@ SYMBOLS = {
     "rtvla_time_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.POINTER(ctypes.c_float)]),
     "rtvla_pretile_elems": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "rtvla_pretile": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P]),
+    "rtvla_linear_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 5),
+    "rtvla_linear": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, ctypes.c_int, _P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, _P]),
+    "rtvla_linear_tile_shape": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
     "rtvla_preprocess_image_scratch": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "rtvla_preprocess_image": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P, ctypes.c_size_t, _P]),
     "rtvla_preprocess_state": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, ctypes.c_int, ctypes.c_int, _P, _P, _P, _P]),

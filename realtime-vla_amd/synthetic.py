@@ -146,9 +146,9 @@ def _sincos_time(t, dim=1024, min_period=4e-3, max_period=4.0):
     return torch.cat([torch.sin(ang), torch.cos(ang)]).to(torch.float32)
 
 
-def pi0_checkpoint(seed, prompt_len, device="cpu", vision_layers=27, llm_layers=18, std=0.02):
+def pi0_checkpoint(seed, prompt_len, device="cpu", vision_layers=27, llm_layers=18, std=0.02, norms="ones"):
     """Synthetic converted Pi0 checkpoint (keys/shapes of /root/reference/pi0_infer.py:1245-1287).
-    Matrices N(0, std^2); LayerNorm weights 1, LayerNorm biases 0."""
+    Matrices N(0, std^2); LayerNorm parameters per `norms` (see _norm_params)."""
     V, L = vision_layers, llm_layers
     shapes = {
         "vision_patch_embedding_w": (14, 14, 3, 1152),
@@ -188,24 +188,29 @@ def pi0_checkpoint(seed, prompt_len, device="cpu", vision_layers=27, llm_layers=
     # (/root/reference/convert_from_jax.py:192-194); the synthetic checkpoint does the same
     for k in ("decoder_action_fused_out_proj_w", "decoder_action_fused_out_proj_b"):
         ck[k] = (ck[k].float() * -0.1).to(torch.bfloat16)
-    _norm_params(ck, V, device)
+    _norm_params(ck, V, device, seed, norms)
     ck["language_embeds"] = language_embeds(seed, prompt_len, device)
     return ck
 
 
-def _norm_params(ck, V, device):
-    one = lambda *s: torch.ones(*s, dtype=torch.bfloat16, device=device)
-    zero = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=device)
-    ck["vision_pre_attn_norm_w"] = one(V, 1152)
-    ck["vision_pre_attn_norm_b"] = zero(V, 1152)
-    ck["vision_pre_ffn_norm_w"] = one(V, 1152)
-    ck["vision_pre_ffn_norm_b"] = zero(V, 1152)
-    ck["vision_final_norm_w"] = one(1152)
-    ck["vision_final_norm_b"] = zero(1152)
+def _norm_params(ck, V, device, seed=0, norms="ones"):
+    """SigLIP LayerNorm parameters.  "ones": weight 1, bias 0 (the benchmark configurations).  "random": every
+    layer's weights 1 + N(0, 0.1^2) and biases N(0, 0.1^2), all distinct, so that the affine term and the choice
+    of the layer's parameters show in the result."""
+    shapes = {"vision_pre_attn_norm": (V, 1152), "vision_pre_ffn_norm": (V, 1152), "vision_final_norm": (1152,)}
+    for name, shape in shapes.items():
+        if norms == "ones":
+            ck[name + "_w"] = torch.ones(*shape, dtype=torch.bfloat16, device=device)
+            ck[name + "_b"] = torch.zeros(*shape, dtype=torch.bfloat16, device=device)
+        elif norms == "random":
+            ck[name + "_w"] = (1.0 + normal_bf16(seed, name + "_w", shape, 0.1, device).float()).to(torch.bfloat16)
+            ck[name + "_b"] = normal_bf16(seed, name + "_b", shape, 0.1, device)
+        else:
+            raise ValueError("norms must be 'ones' or 'random'")
 
 
 def pi05_checkpoint(seed, prompt_len, device="cpu", vision_layers=27, llm_layers=18, std=0.02,
-                    state_tokens=32):
+                    state_tokens=32, norms="ones"):
     """Synthetic converted Pi05 checkpoint (keys/shapes of /root/reference/pi05_infer.py:563-611);
     `decoder_time_embeds` is the closed-form sin/cos embedding of t = 1.0, 0.9, ... 0.1
     (/root/reference/convert_from_jax_pi05.py:214-228)."""
@@ -250,7 +255,7 @@ def pi05_checkpoint(seed, prompt_len, device="cpu", vision_layers=27, llm_layers
         "decoder_final_norm_mod_b": (3072,),
     }
     ck = {k: normal_bf16(seed, k, s, std, device) for k, s in shapes.items()}
-    _norm_params(ck, V, device)
+    _norm_params(ck, V, device, seed, norms)
     te = torch.stack([_sincos_time(1.0 - 0.1 * s) for s in range(10)])
     ck["decoder_time_embeds"] = te.to(torch.bfloat16).to(device)
     ck["language_embeds"] = language_embeds(seed, prompt_len, device, state_tokens=state_tokens)

@@ -99,3 +99,15 @@ def test_workspace_layout(lib):
     assert all(a[1] <= b[0] for a, b in zip(offs, offs[1:])), "workspace regions overlap"
     assert all(v[0] % 256 == 0 for v in bufs.values())
     assert lib.rtvla_pretile_elems(588, 1152) == 72 * 20 * 512
+
+
+def test_unit_entry_points_check_sizes_before_touching_a_device(lib):
+    p = ctypes.c_void_p(4096)
+    assert lib.rtvla_linear_workspace_bytes(768, 1152, 3456, -1, 1) > 768 * 1152 * 2
+    assert lib.rtvla_linear_workspace_bytes(16, 12, 16, -1, 1) == 0                    # K must be a multiple of 8
+    assert lib.rtvla_linear_workspace_bytes(65, 1024, 64, capi.TILE_SKINNY, 1) == 0    # the streaming kernel takes at most 64 rows
+    assert lib.rtvla_linear(p, 16, 128, p, 16, None, p, p, 16, -1, 1, None) == capi.ERR_SIZE
+    assert lib.rtvla_linear(None, 16, 128, p, 16, None, p, p, 1 << 20, -1, 1, None) == 1
+    r, c = ctypes.c_int(), ctypes.c_int()
+    assert lib.rtvla_linear_tile_shape(0, ctypes.byref(r), ctypes.byref(c)) == 0 and (r.value, c.value) == (224, 256)
+    assert lib.rtvla_linear_tile_shape(99, ctypes.byref(r), ctypes.byref(c)) == 1

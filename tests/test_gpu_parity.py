@@ -3,8 +3,17 @@
 Tolerances are the ones the task states for this floating-point path: action MAE <= 1e-2 against
 the bf16-boundary oracle, per-layer relative L2 <= 2e-2.  "Per layer" is measured layer-locally:
 each stage is fed the oracle's input for that layer (teacher forcing) so that the bf16 drift two
-independent pipelines accumulate over 45 layers (3e-2 between the oracle's own bf16 and fp32
-variants) is not charged to any single kernel.  Free-running drift is printed for the record.
+independent pipelines accumulate over 45 layers is not charged to any single kernel.  The
+free-running cumulative drift is bounded as well: at every tap it may not exceed DRIFT_FACTOR times
+the drift between the oracle's own bf16-boundary and all-fp32 variants at that tap (two bf16
+pipelines that round at different places differ from each other by about sqrt(2) times what each
+differs from exact arithmetic), with DRIFT_FLOOR for taps where that figure is a single rounding.
+
+The golden files are written by the oracle itself (tests/golden/make_golden.py): they guard against
+the oracle drifting, they are not an independent anchor.  The oracle's independent pins are
+tests/test_oracle_ops.py and tests/test_oracle_layers.py.  Except for the BASELINE configurations
+C1-C4 (which specify LayerNorm weights of 1), every case here uses random LayerNorm weights and
+biases that differ per layer.
 """
 import os
 
@@ -18,6 +27,8 @@ pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
 MAE_TOL = 1e-2
 LAYER_TOL = 2e-2
+DRIFT_FACTOR = 1.5
+DRIFT_FLOOR = 1e-2
 
 
 def rel(a, b):
@@ -32,7 +43,8 @@ def bf(x, dev="cuda"):
 class Case:
     """One model instance + its oracle run with taps."""
 
-    def __init__(self, model, seed, views, prompt, chunk, vision_layers=27, llm_layers=18, state_tokens=0, max_prompt=None):
+    def __init__(self, model, seed, views, prompt, chunk, vision_layers=27, llm_layers=18, state_tokens=0, max_prompt=None,
+                 norms="random"):
         import rtvla_capi as capi
         from oracle import pi0 as o0, pi05 as o5, ops
         self.capi, self.ops = capi, ops
@@ -41,7 +53,7 @@ class Case:
         dev = "cuda:0"
         if model == "pi0":
             from pi0_infer import Pi0Inference
-            self.ck = syn.pi0_checkpoint(seed, prompt, dev, vision_layers, llm_layers)
+            self.ck = syn.pi0_checkpoint(seed, prompt, dev, vision_layers, llm_layers, norms=norms)
             self.img, self.state, self.noise = syn.observation(seed, views, chunk, dev)
             self.m = Pi0Inference(self.ck, views, chunk)
             self.S_e = 256 * views + prompt
@@ -49,7 +61,7 @@ class Case:
             self.valid = self.S_e
         else:
             from pi05_infer import Pi05Inference
-            self.ck = syn.pi05_checkpoint(seed, prompt, dev, vision_layers, llm_layers, state_tokens=state_tokens)
+            self.ck = syn.pi05_checkpoint(seed, prompt, dev, vision_layers, llm_layers, state_tokens=state_tokens, norms=norms)
             self.img, self.state, self.noise = syn.observation(seed, views, chunk, dev)
             plen = prompt + state_tokens
             if max_prompt is not None and max_prompt != plen:
@@ -64,11 +76,13 @@ class Case:
             self.S_d = chunk
             self.valid = 256 * views + plen
         self.ckc = {k: v.cpu() for k, v in self.ck.items()}
-        self.taps = {}
+        self.taps, self.taps32 = {}, {}
         if model == "pi0":
             self.ref = o0.forward(self.ckc, self.img.cpu(), self.state.cpu(), self.noise.cpu(), taps=self.taps)
+            o0.forward(self.ckc, self.img.cpu(), self.state.cpu(), self.noise.cpu(), bf16_boundaries=False, taps=self.taps32)
         else:
             self.ref = o5.forward(self.ckc, self.img.cpu(), self.noise.cpu(), max_prompt_len=max_prompt, taps=self.taps)
+            o5.forward(self.ckc, self.img.cpu(), self.noise.cpu(), max_prompt_len=max_prompt, bf16_boundaries=False, taps=self.taps32)
         self.e, self.B = self.m._engine, self.m.buffers
         self.keys_pad = self.B["encoder_Vt"].shape[1]
 
@@ -118,29 +132,36 @@ class Case:
     # ---- the checks ----
     def free_running(self):
         """Whole forward stage by stage; returns the drift per tap and the final MAE."""
-        c, t = self.capi, self.taps
+        c, t, t32 = self.capi, self.taps, self.taps32
         self.stage_inputs()
-        drift = {}
+        drift, self.oracle_drift = {}, {}
+
+        def note(name, got, tap, rows=None):
+            a, b = t[tap], t32[tap]
+            if rows is not None:
+                got, a, b = got[:rows], a[:rows], b[:rows]
+            drift[name] = rel(got, a)
+            self.oracle_drift[name] = rel(a, b)
         self.run(c.STAGE_VISION_EMBED)
-        drift["vision_embed"] = rel(self.B["vision_x"], t["vision_embed"])
+        note("vision_embed", self.B["vision_x"], "vision_embed")
         for i in range(self.VL):
             self.run(c.STAGE_VISION_LAYER, i)
-            drift["vision_x/%d" % i] = rel(self.B["vision_x"], t["vision_x/%d" % i])
+            note("vision_x/%d" % i, self.B["vision_x"], "vision_x/%d" % i)
         self.run(c.STAGE_PROJECT)
-        drift["encoder_x0"] = rel(self.B["encoder_x"][: self.valid], t["encoder_x0"][: self.valid])
+        note("encoder_x0", self.B["encoder_x"], "encoder_x0", self.valid)
         for i in range(self.LL):
             self.run(c.STAGE_PREFIX_LAYER, i)
             K, V = self.cache(i)
-            drift["encoder_K/%d" % i] = rel(K[: self.valid], t["encoder_K/%d" % i][: self.valid])
-            drift["encoder_V/%d" % i] = rel(V[: self.valid], t["encoder_V/%d" % i][: self.valid])
+            note("encoder_K/%d" % i, K, "encoder_K/%d" % i, self.valid)
+            note("encoder_V/%d" % i, V, "encoder_V/%d" % i, self.valid)
         self.run(c.STAGE_SUFFIX_INIT)
         for s in range(10):
             self.run(c.STAGE_SUFFIX_STEP_BEGIN, 0, s)
             for i in range(self.LL):
                 self.run(c.STAGE_SUFFIX_LAYER, i, s)
-            drift["decoder_x/%d" % s] = rel(self.dec_x(), t["decoder_x/%d/%d" % (s, self.LL - 1)])
+            note("decoder_x/%d" % s, self.dec_x(), "decoder_x/%d/%d" % (s, self.LL - 1))
             self.run(c.STAGE_SUFFIX_STEP_END, 0, s)
-            drift["noise/%d" % s] = rel(self.B["diffusion_noise"], t["noise/%d" % s])
+            note("noise/%d" % s, self.B["diffusion_noise"], "noise/%d" % s)
         out = self.B["diffusion_noise"].float().cpu().clone()
         return drift, out
 
@@ -195,9 +216,13 @@ def check_case(case, gold_key=None, gold_file="golden_small.pt"):
     drift, staged = case.free_running()
     mae = (staged - case.ref).abs().mean().item()
     worst = max(drift, key=drift.get)
-    print("\n[%s] free-running: action MAE %.5f, largest cumulative rel-L2 %.4f at %s" % (gold_key, mae, drift[worst], worst))
+    bound = {k: max(DRIFT_FACTOR * case.oracle_drift[k], DRIFT_FLOOR) for k in drift}
+    tight = max(drift, key=lambda k: drift[k] / bound[k])
+    print("\n[%s] free-running: action MAE %.5f, largest cumulative rel-L2 %.4f at %s (oracle bf16 vs fp32 there: %.4f); "
+          "closest to its bound: %s at %.2f of it" % (gold_key, mae, drift[worst], worst, case.oracle_drift[worst], tight, drift[tight] / bound[tight]))
     assert torch.isfinite(staged).all()
     assert mae <= MAE_TOL
+    assert drift[tight] <= bound[tight], (tight, drift[tight], bound[tight])
     per_dim = (staged - case.ref).abs().mean(0)
     assert per_dim.max().item() <= 3 * MAE_TOL          # per-dimension MAE, the second statistic of test.py:282-287
     out = case.forward().float().cpu()                    # the captured graph, same inputs
@@ -254,11 +279,18 @@ def test_shape_sweep_against_the_oracle(model, views, prompt, chunk, state_token
     ("c3", ("pi0", 1234, 3, 0, 63)),
 ])
 def test_pi0_full_size_configs(name, spec):
-    check_case(Case(*spec), name, "golden_full.pt")
+    check_case(Case(*spec, norms="ones"), name, "golden_full.pt")         # the BASELINE configurations specify norms = 1
 
 
 def test_pi05_full_size_c4():
-    check_case(Case("pi05", 1234, 3, 20, 50, state_tokens=32), "c4", "golden_full.pt")
+    check_case(Case("pi05", 1234, 3, 20, 50, state_tokens=32, norms="ones"), "c4", "golden_full.pt")
+
+
+def test_pi0_full_size_headline_shape_with_random_norms():
+    """The shape the headline metric is quoted on (3 views, 20-token prompt, chunk 50) at full depth, with LayerNorm
+    weights and biases that are random and distinct per layer: every per-layer parameter pick of the 27 SigLIP layers
+    and the final norm shows in the taps."""
+    check_case(Case("pi0", 1234, 3, 20, 50, norms="random"), "headline", "golden_full.pt")
 
 
 def test_c5_prefix_stress_sustained_replay():

@@ -13,14 +13,14 @@ GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "golden_small.pt")
 
 @pytest.fixture(scope="module")
 def small_pi0():
-    ck = syn.pi0_checkpoint(7, 4, vision_layers=2, llm_layers=2)
+    ck = syn.pi0_checkpoint(7, 4, vision_layers=2, llm_layers=2, norms="random")
     img, st, nz = syn.observation(7, 1, 10)
     return ck, img, st, nz
 
 
 @pytest.fixture(scope="module")
 def small_pi05():
-    ck = syn.pi05_checkpoint(9, 4, vision_layers=2, llm_layers=2, state_tokens=3)
+    ck = syn.pi05_checkpoint(9, 4, vision_layers=2, llm_layers=2, state_tokens=3, norms="random")
     img, _, nz = syn.observation(9, 1, 10)
     return ck, img, nz
 
@@ -112,9 +112,12 @@ def test_pi05_is_independent_of_prefix_padding(small_pi05):
     """Rows past the valid prompt length are masked as keys and never read as queries, and the
     suffix RoPE offset follows the valid length: the allocation size must not change the result."""
     ck, img, nz = small_pi05
+    a = pi05.forward(ck, img, nz, max_prompt_len=7, bf16_boundaries=False)
+    b = pi05.forward(ck, img, nz, max_prompt_len=19, bf16_boundaries=False)
+    assert torch.allclose(a, b, atol=1e-5)                 # (the CPU BLAS sums in a shape-dependent order, hence not bit-equal)
     a = pi05.forward(ck, img, nz, max_prompt_len=7)
     b = pi05.forward(ck, img, nz, max_prompt_len=19)
-    assert torch.equal(a, b)
+    assert (a - b).abs().mean().item() < 1e-4 and (a != b).float().mean().item() < 0.05      # a few single-ulp flips at most
 
 
 def test_pi05_zero_gate_freezes_the_residual_stream(small_pi05):
@@ -150,7 +153,7 @@ def test_adarms_reduces_to_rms_norm_with_zero_style():
 
 
 def test_pi0_runs_with_an_empty_prompt():
-    ck = syn.pi0_checkpoint(8, 0, vision_layers=1, llm_layers=2)
+    ck = syn.pi0_checkpoint(8, 0, vision_layers=1, llm_layers=2, norms="random")
     img, st, nz = syn.observation(8, 1, 63)
     out = pi0.forward(ck, img, st, nz)
     g = torch.load(GOLDEN, weights_only=True)
