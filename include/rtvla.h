@@ -197,6 +197,17 @@ size_t rtvla_preprocess_image_scratch(int height, int width);
 int rtvla_preprocess_image(const void* src_u8, int height, int width, void* dst_bf16, void* scratch, size_t scratch_bytes,
                            void* hip_stream);
 
+/* The same computation for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The 8-bit
+ * intermediate lives in a device array that is part of the library's code object (RTVLA_STATIC_SCRATCH_BYTES, held by
+ * every GPU the library is loaded on until the process ends); the call allocates nothing.  Frames whose intermediate
+ * (height x resized width x 3 bytes, resized width <= 224) exceeds that size - more than 2160 rows at full width - are
+ * rejected with RTVLA_ERR_LIMIT before anything is enqueued.  All calls on one GPU share the one array: calls that
+ * overlap on the same GPU (different streams or threads) race; calls on one stream are ordered.  Nothing in the array
+ * has to start at zero: the horizontal pass writes every byte the vertical pass reads. */
+#define RTVLA_STATIC_SCRATCH_BYTES (2160 * 224 * 3)
+int rtvla_preprocess_image_static(const void* src_u8, int height, int width, void* dst_bf16, void* hip_stream);
+
 /* Replaces _normalize_state (+ _digitize_state) (test.py:121-137): state[n] and the statistics [n_stats] are
  * zero-padded to 32 like _pad_to_dim; mode 0 (Pi0): (x - a) / (b + 1e-6) with a = mean, b = std; mode 1 (Pi05):
  * (x - a) / (b - a + 1e-6) * 2 - 1 with a = q01, b = q99, all in double as numpy computes it.  Outputs (each may

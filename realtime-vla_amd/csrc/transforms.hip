@@ -12,6 +12,12 @@
 #include "../../include/rtvla.h"
 #include "common.h"
 #include <math.h>
+#include <mutex>
+
+// 8-bit intermediate of the horizontal pass for rtvla_preprocess_image_static: part of the code object, so every
+// GPU the library runs on holds its own copy at its own address from load until the process ends.  Host code
+// never passes this name to a kernel; it uses the per-device address resolved in static_scratch_ptr().
+static __device__ __align__(256) unsigned char scratch[RTVLA_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -127,17 +133,12 @@ __global__ void actions_kernel(const bf16_t* __restrict__ actions, int chunk, co
     out[idx] = v;
 }
 
-}  // namespace
-
-extern "C" {
-
-size_t rtvla_preprocess_image_scratch(int height, int width) {
-    if (height <= 0 || width <= 0) return 0;
-    return ((size_t)height * 224 * 3 + 255) & ~(size_t)255;       // the horizontal pass never produces more than 224 columns
-}
-
-int rtvla_preprocess_image(const void* src_u8, int height, int width, void* dst_bf16, void* scratch, size_t scratch_bytes, void* stream) {
-    if (!src_u8 || !dst_bf16 || !scratch || height <= 0 || width <= 0) return RTVLA_ERR_ARG;
+// geometry, limits and the two launches shared by rtvla_preprocess_image and rtvla_preprocess_image_static;
+// `get_scratch` is asked for the intermediate buffer only after every size check has passed
+template <typename GetScratch>
+int preprocess_image_impl(const void* src_u8, int height, int width, void* dst_bf16, size_t scratch_bytes, int too_small_code,
+                          GetScratch get_scratch, void* stream) {
+    if (!src_u8 || !dst_bf16 || height <= 0 || width <= 0) return RTVLA_ERR_ARG;
     // geometry of test.py:105-116 (Python float arithmetic = C double arithmetic)
     int rh = 224, rw = 224, pad_top = 0, pad_left = 0;
     if (!(width == 224 && height == 224)) {
@@ -150,13 +151,52 @@ int rtvla_preprocess_image(const void* src_u8, int height, int width, void* dst_
     if (rh < 1 || rw < 1 || rh > 224 || rw > 224) return RTVLA_ERR_ARG;
     const double sx = (double)width / rw, sy = (double)height / rh;
     if ((int)ceil(sx > 1.0 ? sx : 1.0) * 2 + 1 > MAX_TAPS || (int)ceil(sy > 1.0 ? sy : 1.0) * 2 + 1 > MAX_TAPS) return RTVLA_ERR_LIMIT;
-    if (scratch_bytes < (size_t)height * rw * 3) return RTVLA_ERR_SIZE;
+    if (scratch_bytes < (size_t)height * rw * 3) return too_small_code;
+    uint8_t* tmp = nullptr;
+    if (int rc = get_scratch(&tmp)) return rc;
     hipStream_t s = (hipStream_t)stream;
     const int n1 = height * rw;
-    hipLaunchKernelGGL(resample_h_kernel, dim3((n1 + 255) / 256), dim3(256), 0, s, (const uint8_t*)src_u8, height, width, rw, (uint8_t*)scratch);
-    hipLaunchKernelGGL(resample_v_pad_norm_kernel, dim3((224 * 224 + 255) / 256), dim3(256), 0, s, (const uint8_t*)scratch, height, rw, rh,
+    hipLaunchKernelGGL(resample_h_kernel, dim3((n1 + 255) / 256), dim3(256), 0, s, (const uint8_t*)src_u8, height, width, rw, tmp);
+    hipLaunchKernelGGL(resample_v_pad_norm_kernel, dim3((224 * 224 + 255) / 256), dim3(256), 0, s, (const uint8_t*)tmp, height, rw, rh,
                        pad_top, pad_left, (bf16_t*)dst_bf16);
     return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
+}
+
+// Device address of `scratch` on the current device, resolved once per device with that device current.
+constexpr int MAX_DEVICES = 64;
+std::mutex static_scratch_mutex;
+void* static_scratch_addr[MAX_DEVICES] = {};
+
+int static_scratch_ptr(uint8_t** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return RTVLA_ERR_DEVICE;
+    std::lock_guard<std::mutex> lock(static_scratch_mutex);
+    if (!static_scratch_addr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return RTVLA_ERR_DEVICE;
+        static_scratch_addr[dev] = ptr;
+    }
+    *out = (uint8_t*)static_scratch_addr[dev];
+    return RTVLA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t rtvla_preprocess_image_scratch(int height, int width) {
+    if (height <= 0 || width <= 0) return 0;
+    return ((size_t)height * 224 * 3 + 255) & ~(size_t)255;       // the horizontal pass never produces more than 224 columns
+}
+
+int rtvla_preprocess_image(const void* src_u8, int height, int width, void* dst_bf16, void* scratch_arg, size_t scratch_bytes, void* stream) {
+    if (!scratch_arg) return RTVLA_ERR_ARG;
+    return preprocess_image_impl(src_u8, height, width, dst_bf16, scratch_bytes, RTVLA_ERR_SIZE,
+                                 [&](uint8_t** out) { *out = (uint8_t*)scratch_arg; return (int)RTVLA_OK; }, stream);
+}
+
+int rtvla_preprocess_image_static(const void* src_u8, int height, int width, void* dst_bf16, void* stream) {
+    return preprocess_image_impl(src_u8, height, width, dst_bf16, (size_t)RTVLA_STATIC_SCRATCH_BYTES, RTVLA_ERR_LIMIT, static_scratch_ptr, stream);
 }
 
 int rtvla_preprocess_state(const double* state, int n, const double* stat_a, const double* stat_b, int n_stats, int mode,

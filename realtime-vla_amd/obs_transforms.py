@@ -52,15 +52,24 @@ class ObservationTransforms:
             image = image.permute(1, 2, 0)
         return image.to(self.device).contiguous()
 
-    def resize_pad_normalize_into(self, image, out_view):
+    def resize_pad_normalize_into(self, image, out_view, static_scratch=False):
         """_resize_with_pad + _normalize_image of one image into out_view (bf16 [224, 224, 3], e.g. one view of the
-        model's observation_images_normalized buffer)."""
+        model's observation_images_normalized buffer).  With static_scratch the library's built-in intermediate buffer
+        is used and nothing is allocated (frames of at most 2160 rows at full width; calls on one GPU must not overlap)."""
         img = self._parse_image(image)
         h, w, c = img.shape
         if c != 3 or img.dtype != torch.uint8:
             raise ValueError("expected an RGB uint8 image, got shape %s dtype %s" % (tuple(img.shape), img.dtype))
         if out_view.dtype != torch.bfloat16 or tuple(out_view.shape) != (224, 224, 3) or not out_view.is_contiguous():
             raise ValueError("out_view must be a contiguous bf16 [224, 224, 3] tensor")
+        if static_scratch:
+            rc = self.lib.rtvla_preprocess_image_static(_P(img.data_ptr()), h, w, _P(out_view.data_ptr()), self._stream())
+            if rc == capi.ERR_LIMIT:
+                raise ValueError("a %d x %d frame does not fit the library's %d-byte static intermediate buffer (or shrinks by more "
+                                 "than a factor of 31)" % (h, w, capi.STATIC_SCRATCH_BYTES))
+            self._check(rc, "rtvla_preprocess_image_static")
+            self._keep = img
+            return out_view
         need = self.lib.rtvla_preprocess_image_scratch(h, w)
         if self._scratch.numel() < need:
             self._scratch = torch.empty(need, dtype=torch.uint8, device=self.device)

@@ -22,6 +22,7 @@ STAGE_SUFFIX_STEP_END = 7
 
 ERR_NAME, ERR_SIZE, ERR_STATE, ERR_LIMIT = 2, 3, 4, 7
 TILE_AUTO, TILE_SKINNY = -1, -2
+STATIC_SCRATCH_BYTES = 2160 * 224 * 3          # RTVLA_STATIC_SCRATCH_BYTES
 
 
 class Dims(ctypes.Structure):
@@ -65,6 +66,7 @@ SYMBOLS = {
     "rtvla_linear_tile_shape": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
     "rtvla_preprocess_image_scratch": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "rtvla_preprocess_image": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P, ctypes.c_size_t, _P]),
+    "rtvla_preprocess_image_static": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P]),
     "rtvla_preprocess_state": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, ctypes.c_int, ctypes.c_int, _P, _P, _P, _P]),
     "rtvla_postprocess_actions": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, ctypes.c_int, ctypes.c_int, _P, ctypes.c_int, _P, _P]),
 }

@@ -101,7 +101,7 @@ def test_workspace_layout(lib):
     assert lib.rtvla_pretile_elems(588, 1152) == 72 * 20 * 512
 
 
-def test_unit_entry_points_check_sizes_before_touching_a_device(lib):
+def test_unit_and_static_entry_points_check_sizes_before_touching_a_device(lib):
     p = ctypes.c_void_p(4096)
     assert lib.rtvla_linear_workspace_bytes(768, 1152, 3456, -1, 1) > 768 * 1152 * 2
     assert lib.rtvla_linear_workspace_bytes(16, 12, 16, -1, 1) == 0                    # K must be a multiple of 8
@@ -111,3 +111,8 @@ def test_unit_entry_points_check_sizes_before_touching_a_device(lib):
     r, c = ctypes.c_int(), ctypes.c_int()
     assert lib.rtvla_linear_tile_shape(0, ctypes.byref(r), ctypes.byref(c)) == 0 and (r.value, c.value) == (224, 256)
     assert lib.rtvla_linear_tile_shape(99, ctypes.byref(r), ctypes.byref(c)) == 1
+    # the allocation-free image entry point: a frame whose intermediate exceeds the static buffer is refused up front
+    assert lib.rtvla_preprocess_image_static(p, 2400, 2400, p, None) == capi.ERR_LIMIT
+    assert lib.rtvla_preprocess_image_static(p, 8000, 250, p, None) == capi.ERR_LIMIT  # shrink factor above 31
+    assert lib.rtvla_preprocess_image_static(None, 10, 10, p, None) == 1
+    assert capi.STATIC_SCRATCH_BYTES == 2160 * 224 * 3
