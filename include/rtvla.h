@@ -143,9 +143,10 @@ int rtvla_graph_launch(rtvla_ctx* ctx, void* hip_stream);
 /* Number of kernels the last forward (or stage) enqueued: the kernel nodes of the captured graph. */
 int rtvla_launch_count(const rtvla_ctx* ctx);
 
-/* Measurement helper (no reference counterpart): run `stage` `iters` times back to back on the
- * stream between two HIP events recorded on that same stream and return the mean milliseconds
- * per run.  With layer = -1 every layer of the stage runs in turn (weights cold, as inside a forward) and the
+/* Measurement helper (no reference counterpart): record `stage` `iters` times back to back into a temporary HIP
+ * graph, replay it on the stream between two HIP events recorded on that same stream and return the mean
+ * milliseconds per run (a graph, because the forward runs as one and eager launches of microsecond kernels would
+ * measure the host's launch rate).  With layer = -1 every layer of the stage runs in turn (weights cold, as inside a forward) and the
  * mean is per layer.  Synchronises the stream. */
 int rtvla_time_stage(rtvla_ctx* ctx, int stage, int layer, int step, int iters, void* hip_stream, float* mean_ms);
 

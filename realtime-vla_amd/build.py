@@ -1,4 +1,5 @@
-"""Build librtvla.so (gfx950) in-tree with hipcc: python build.py [--force]."""
+"""Build librtvla.so (gfx950) in-tree with hipcc: python build.py [-v] [-DNAME ...] [-o OUT.so]
+(-D / -o make a variant build, e.g. -DRTVLA_TUNING with its environment knobs, next to the shipped library)."""
 import os
 import subprocess
 import sys
@@ -21,9 +22,10 @@ def _hipcc():
     return "hipcc"
 
 
-def _compile(src):
-    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [_hipcc()] + FLAGS + EXTRA.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(job):
+    src, defines, tag = job
+    obj = os.path.join(CSRC, src.replace(".hip", tag + ".o"))
+    cmd = [_hipcc()] + FLAGS + list(defines) + EXTRA.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "warnings generated" not in l)
     if r.returncode != 0:
@@ -31,22 +33,25 @@ def _compile(src):
     return obj, err
 
 
-def build(force=True, verbose=False):
+def build(force=True, verbose=False, defines=(), out=LIB):
     """Compile every HIP source for gfx950 and link the shared library."""
-    if not force and os.path.exists(LIB):
-        return LIB
+    if not force and os.path.exists(out):
+        return out
+    tag = "" if out == LIB else "." + os.path.splitext(os.path.basename(out))[0]
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4)) as ex:
-        results = list(ex.map(_compile, SOURCES))
+        results = list(ex.map(_compile, [(src, defines, tag) for src in SOURCES]))
     if verbose:
         for _, err in results:
             if err.strip():
                 print(err)
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + [o for o, _ in results]
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + [o for o, _ in results]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
-    return LIB
+    return out
 
 
 if __name__ == "__main__":
-    print(build(force=True, verbose="-v" in sys.argv))
+    argv = sys.argv[1:]
+    out = os.path.abspath(argv[argv.index("-o") + 1]) if "-o" in argv else LIB
+    print(build(force=True, verbose="-v" in argv, defines=[a for a in argv if a.startswith("-D")], out=out))

@@ -7,6 +7,17 @@
 #include <stdint.h>
 #include "common.h"
 
+// Tuning builds (-DRTVLA_TUNING) can knock parts of a kernel out at run time (environment variable RTVLA_KO, a bit
+// mask read at launch) to attribute its time; in the shipped build KO() is constant false and the field does not exist.
+#ifdef RTVLA_TUNING
+#define RTVLA_KO_FIELD int ko;
+#define KO(p, bit) (((p).ko & (bit)) != 0)
+int rtvla_tuning_ko();
+#else
+#define RTVLA_KO_FIELD
+#define KO(p, bit) false
+#endif
+
 // ----- pre-tiled weights ------------------------------------------------------------
 // A weight W[K][N] (row-major, "in x out") is re-laid out once as MFMA operand fragments:
 // tile (nb, kb) holds the 16 columns nb*16.. and 32 rows kb*32.. as 64 lanes x 8 bf16,
@@ -86,6 +97,7 @@ struct SkinnyP {
     const bf16_t* bias; const bf16_t* gate;    // per-column
     const bf16_t* rope;                        // [row][256]
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt; int kv_row0;
+    RTVLA_KO_FIELD
 };
 int launch_skinny(const SkinnyP& p, int epi, hipStream_t s);
 
@@ -110,6 +122,7 @@ struct AttnP {
     // key split over workgroups (nsplit > 1, at most 16): fp32 partial records, combined by a second launch
     int nsplit; float* partial; size_t partial_floats;
     int kb_per_split, nsplit_eff;    // filled by the launcher
+    RTVLA_KO_FIELD
 };
 enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1 };    // many rows, two row tiles per workgroup / few rows, one row tile and a key split
 int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s);

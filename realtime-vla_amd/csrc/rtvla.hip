@@ -12,6 +12,10 @@
 #include <string>
 #include <vector>
 
+#ifdef RTVLA_TUNING
+int rtvla_tuning_ko() { const char* e = getenv("RTVLA_KO"); return e ? atoi(e) : 0; }
+#endif
+
 namespace {
 
 struct Tensor {
@@ -51,6 +55,7 @@ struct rtvla_ctx {
     bool prepared = false;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    hipStream_t timing_stream = nullptr;     // the measurement helpers capture graphs, which the null stream cannot
     std::string err;
     int launches = 0;              // scheduler launches enqueued so far (index space of rtvla_time_launch)
     int kernels = 0;               // kernels behind them (the key-split attention is two)
@@ -625,6 +630,7 @@ int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out) {
 int rtvla_destroy(rtvla_ctx* c) {
     if (!c) return RTVLA_ERR_ARG;
     drop_graph(c);
+    if (c->timing_stream) hipStreamDestroy(c->timing_stream);
     delete c;
     return RTVLA_OK;
 }
@@ -743,71 +749,79 @@ int rtvla_graph_launch(rtvla_ctx* c, void* stream) {
 
 int rtvla_launch_count(const rtvla_ctx* c) { return c ? c->kernels : 0; }
 
-int rtvla_time_stage(rtvla_ctx* c, int stage, int layer, int step, int iters, void* stream, float* mean_ms) {
-    if (int rc = check_ready(c, true)) return rc;
-    if (iters < 1 || !mean_ms) return RTVLA_ERR_ARG;
-    hipStream_t s = (hipStream_t)stream;
-    hipEvent_t a, b;
-    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
+// Both measurement helpers record their launches into a temporary HIP graph and time one replay of it with events on
+// the stream: back-to-back eager launches of kernels that last a few microseconds would measure the host's launch
+// rate, not the kernels, and the forward itself runs as a graph.
+static int time_replay(rtvla_ctx* c, hipStream_t s, int stage, int layer, int step, int launch_index, int iters, float* mean_ms, int* enqueued_out) {
+    if (!s) {
+        // the null stream cannot be captured: finish what it holds, then launch and time on a stream of the context's own
+        hipError_t e0 = hipStreamSynchronize(nullptr);
+        if (e0 == hipSuccess && !c->timing_stream) e0 = hipStreamCreateWithFlags(&c->timing_stream, hipStreamNonBlocking);
+        if (e0 != hipSuccess) return hip_fail(c, e0, "timing stream");
+        s = c->timing_stream;
+    }
     Sched sc(c, s);
-    c->status = 0;
-    // layer -1: every layer of the stage in turn (weights cold, as inside a forward), mean per layer
     const bool cycle = layer == -1;
     const int n_layers = !cycle ? 1 : (stage == RTVLA_STAGE_VISION_LAYER ? c->d.vision_layers :
                                        (stage == RTVLA_STAGE_PREFIX_LAYER || stage == RTVLA_STAGE_SUFFIX_LAYER) ? c->d.llm_layers : 1);
     const int first = cycle ? 0 : layer;
-    int rc = sc.stage(stage, first, step);      // warm-up
+    c->status = 0; c->only = launch_index; c->last_name.clear();
+    c->launches = 0; c->kernels = 0;
+    int rc = sc.stage(stage, first, step);      // eager warm-up: sets kernel attributes outside the capture, tells whether the index exists
+    if (!rc && launch_index >= 0 && c->launches <= launch_index) rc = c->fail(RTVLA_ERR_ARG, "launch index past the end of the stage");
+    if (rc) { c->only = -1; return rc; }
+    hipError_t e = hipStreamSynchronize(s);
+    if (e != hipSuccess) { c->only = -1; return hip_fail(c, e, "warm-up launch"); }
+    hipGraph_t g = nullptr; hipGraphExec_t ge = nullptr;
+    e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) { c->only = -1; return hip_fail(c, e, "hipStreamBeginCapture"); }
+    int enqueued = 0;
+    for (int i = 0; i < iters && !rc; ++i)
+        for (int l = first; l < first + n_layers && !rc; ++l) {
+            c->launches = 0; c->kernels = 0;
+            rc = sc.stage(stage, l, step);
+            enqueued += launch_index < 0 ? 1 : (c->launches > launch_index);          // (the last prefix layer has fewer launches)
+        }
+    e = hipStreamEndCapture(s, &g);
+    c->only = -1;
+    if (e != hipSuccess) return hip_fail(c, e, "hipStreamEndCapture");
+    if (!rc && c->status) rc = c->status;
+    if (!rc) { e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0); if (e != hipSuccess) rc = hip_fail(c, e, "hipGraphInstantiate"); }
+    hipEvent_t a = nullptr, b = nullptr;
+    if (!rc && (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess)) rc = c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
     if (!rc) {
+        hipGraphLaunch(ge, s);                  // one untimed replay
         hipEventRecord(a, s);
-        for (int i = 0; i < iters && !rc; ++i)
-            for (int l = first; l < first + n_layers && !rc; ++l) rc = sc.stage(stage, l, step);
+        hipGraphLaunch(ge, s);
         hipEventRecord(b, s);
-        hipError_t e = hipEventSynchronize(b);
-        if (e != hipSuccess) rc = hip_fail(c, e, "time_stage");
-        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / (iters * n_layers); }
+        e = hipEventSynchronize(b);
+        if (e != hipSuccess) rc = hip_fail(c, e, "timed replay");
+        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / (enqueued > 0 ? enqueued : 1); }
     }
-    hipEventDestroy(a); hipEventDestroy(b);
-    if (rc) return rc;
-    return c->status;
+    if (a) hipEventDestroy(a);
+    if (b) hipEventDestroy(b);
+    if (ge) hipGraphExecDestroy(ge);
+    if (g) hipGraphDestroy(g);
+    if (enqueued_out) *enqueued_out = enqueued;
+    return rc;
+}
+
+int rtvla_time_stage(rtvla_ctx* c, int stage, int layer, int step, int iters, void* stream, float* mean_ms) {
+    if (int rc = check_ready(c, true)) return rc;
+    if (iters < 1 || !mean_ms) return RTVLA_ERR_ARG;
+    // layer -1: every layer of the stage in turn (weights cold, as inside a forward), mean per layer
+    return time_replay(c, (hipStream_t)stream, stage, layer, step, -1, iters, mean_ms, nullptr);
 }
 
 int rtvla_time_launch(rtvla_ctx* c, int stage, int layer, int step, int launch_index, int iters, void* stream,
                       float* mean_ms, char* name_out, size_t name_cap) {
     if (int rc = check_ready(c, true)) return rc;
     if (iters < 1 || !mean_ms || launch_index < 0) return RTVLA_ERR_ARG;
-    hipStream_t s = (hipStream_t)stream;
-    hipEvent_t a, b;
-    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
-    Sched sc(c, s);
-    c->status = 0; c->only = launch_index; c->last_name.clear();
-    c->launches = 0; c->kernels = 0;
     // layer -1: one launch per layer in turn, so that every launch streams weights nobody has touched since the
     // previous pass (what the kernel sees inside a forward); otherwise the same layer over and over (cache-warm)
-    const bool cycle = layer == -1;
-    const int n_layers = !cycle ? 1 : (stage == RTVLA_STAGE_VISION_LAYER ? c->d.vision_layers :
-                                       (stage == RTVLA_STAGE_PREFIX_LAYER || stage == RTVLA_STAGE_SUFFIX_LAYER) ? c->d.llm_layers : 1);
-    const int first = cycle ? 0 : layer;
-    int rc = sc.stage(stage, first, step);      // warm-up, also tells whether the index exists
-    if (!rc && c->launches <= launch_index) rc = c->fail(RTVLA_ERR_ARG, "launch index past the end of the stage");
-    if (!rc) {
-        int enqueued = 0;
-        hipEventRecord(a, s);
-        for (int i = 0; i < iters && !rc; ++i)
-            for (int l = first; l < first + n_layers && !rc; ++l) {
-                c->launches = 0; c->kernels = 0;
-                rc = sc.stage(stage, l, step);
-                enqueued += c->launches > launch_index;          // (the last prefix layer has fewer launches)
-            }
-        hipEventRecord(b, s);
-        hipError_t e = hipEventSynchronize(b);
-        if (e != hipSuccess) rc = hip_fail(c, e, "time_launch");
-        else { float ms = 0.f; hipEventElapsedTime(&ms, a, b); *mean_ms = ms / (enqueued > 0 ? enqueued : 1); }
-    }
-    c->only = -1;
-    hipEventDestroy(a); hipEventDestroy(b);
+    const int rc = time_replay(c, (hipStream_t)stream, stage, layer, step, launch_index, iters, mean_ms, nullptr);
     if (name_out && name_cap) { strncpy(name_out, c->last_name.c_str(), name_cap - 1); name_out[name_cap - 1] = 0; }
-    if (rc) return rc;
-    return c->status;
+    return rc;
 }
 
 int rtvla_time_forward(rtvla_ctx* c, int iters, void* stream, float* ms_out) {
