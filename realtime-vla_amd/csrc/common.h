@@ -33,11 +33,14 @@ RTVLA_DEVICE bf16x4 pack4(f32x4 v) { return pack4(v[0], v[1], v[2], v[3]); }
 RTVLA_DEVICE bf16x4 load4(const bf16_t* p) { return *(const bf16x4*)p; }
 RTVLA_DEVICE void store4(bf16_t* p, bf16x4 v) { *(bf16x4*)p = v; }
 
-// hardware reciprocal (1 ulp) instead of an IEEE division: the result is rounded to bf16 anyway
-RTVLA_DEVICE float sigmoidf_fast(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
-// tanh-approximated GELU written as a * sigmoid(2 sqrt(2/pi) (a + 0.044715 a^3))
+// hardware reciprocal and base-2 exponential (1 ulp each) instead of an IEEE division and expf: two transcendental
+// instructions and no range fix-ups; the result is rounded to bf16 anyway.  exp2 saturates to 0 / inf, so the
+// sigmoid is exactly 1 / 0 at the far ends and never NaN for finite input.
+RTVLA_DEVICE float sigmoidf_fast(float x) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x)); }
+// tanh-approximated GELU written as a * sigmoid(2 sqrt(2/pi) (a + 0.044715 a^3)), the constants pre-multiplied by -log2(e)
 RTVLA_DEVICE float gelu_tanh(float a) {
-    return a * sigmoidf_fast(1.5957691216057308f * a * (1.0f + 0.044715f * a * a));
+    const float w = a * (-2.3022081981462776f + -0.10294323958057285f * (a * a));
+    return a * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(w));
 }
 RTVLA_DEVICE float siluf(float a) { return a * sigmoidf_fast(a); }
 

@@ -21,27 +21,18 @@ RTVLA_DEVICE f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdg
 
 // MT, NT: 32-row tiles per workgroup and 32-column tiles per wave.  Small tiles are compiled to fit two
 // workgroups per CU so that one workgroup's MFMAs run under the other's memory latency.
+// One block tile of MT 32-row tiles starting at row m0: K loop and epilogue.
 template <int WN, int MT, int NT, int EPI>
-__global__ __launch_bounds__(WN * 64, (MT <= 2 && WN == 4 ? 2 : 1))
-void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int stages_per_split) {
+RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, int n_blk, int split, int stages_total, int stages_per_split) {
     constexpr int NTH = WN * 64;
     constexpr int BM = MT * 32;
     constexpr int A_CHUNKS = BM * 8;                       // 16-byte chunks per 64-wide K stage
     constexpr int AIT = (A_CHUNKS + NTH - 1) / NTH;
     constexpr int STAGE_ELEMS = BM * 64;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     bf16_t* lds = (bf16_t*)smem_raw;
 
     const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
     const int h = lane >> 5, r = lane & 31;
-
-    const int total = m_blocks * n_blocks * p.nsplit;
-    const int lid = xcd_remap(blockIdx.x, total);
-    const int split = lid / (m_blocks * n_blocks);
-    const int rem = lid - split * (m_blocks * n_blocks);
-    const int n_blk = rem / m_blocks;
-    const int m_blk = rem - n_blk * m_blocks;
-    const int m0 = m_blk * BM;
     const int s_begin = split * stages_per_split;
     const int s_end = min(s_begin + stages_per_split, stages_total);
 
@@ -146,7 +137,7 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
             if (t >= HR - AIT) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                  // LDS writes of stage t+1
         }
         __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
+        if (!KO(p, 2)) __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         // ---- second k half ----
         load_b_half(s_next, br, 0);
@@ -196,6 +187,17 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         }
     }
     __syncthreads();                                        // the epilogue reuses the stage buffers
+    if (KO(p, 1)) {                                         // (KO 1: no epilogue; the accumulators stay live through a store that never happens)
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) t += acc[i][j][e];
+        if (t == 1.2345e-30f) p.out[0] = f2bf(t);
+        return;
+    }
 
     // ---- epilogue: lane (h, r) holds rows m = m0 + 32 i + r, columns n = 32 tile + 8 grp + 4 h + e ----
     // Row-major outputs go through LDS one 32-row tile at a time so that the global stores are whole
@@ -211,9 +213,17 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
         unsigned char* obuf = smem_raw;
         const int nbase = n_blk * OUTW;
         const int ncols = p.N16 * 16;
+        // As many 32-row tiles as fit into the stage buffers are converted and staged back to back, then copied out
+        // back to back: one barrier pair per group instead of one per tile, and the stores of a group stream.
+        constexpr int TILE_B = 32 * ROWB;
+        constexpr int GROUP = (3 * BM * 128) / TILE_B >= MT ? MT : ((3 * BM * 128) / TILE_B < 1 ? 1 : (3 * BM * 128) / TILE_B);
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
+        for (int g0 = 0; g0 < MT; g0 += GROUP) {
+#pragma unroll
+          for (int i = g0; i < (g0 + GROUP < MT ? g0 + GROUP : MT); ++i) {
+            if (m0 + i * 32 >= p.M) continue;                                     // a row tile past the end (uniform)
             const int m = m0 + i * 32 + r;
+            unsigned char* const tbuf = obuf + (i - g0) * TILE_B;
 #pragma unroll
             for (int j = 0; j < HALF; ++j) {
 #pragma unroll
@@ -221,11 +231,13 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
                     const int cl = (wn * HALF + j) * 32 + 8 * grp + 4 * h;        // column inside the workgroup tile
                     const int n0 = min(nbase + cl, ncols - 4);                    // clamped: out-of-range columns are never copied out
                     f32x4 v = {acc[i][j][4 * grp], acc[i][j][4 * grp + 1], acc[i][j][4 * grp + 2], acc[i][j][4 * grp + 3]};
-                    unsigned char* dst = obuf + r * ROWB + cl * ESZ;
+                    unsigned char* dst = tbuf + r * ROWB + cl * ESZ;
                     if constexpr (EPI == EPI_PARTIAL) {
                         *(f32x4*)dst = v;
                     } else if constexpr (EPI == EPI_GEGLU) {
                         const f32x4 u = {acc[i][j + HALF][4 * grp], acc[i][j + HALF][4 * grp + 1], acc[i][j + HALF][4 * grp + 2], acc[i][j + HALF][4 * grp + 3]};
+                        if (KO(p, 4)) *(bf16x4*)dst = pack4(v[0] * u[0], v[1] * u[1], v[2] * u[2], v[3] * u[3]);      // (KO 4: no GELU)
+                        else
                         *(bf16x4*)dst = pack4(gelu_tanh(v[0]) * u[0], gelu_tanh(v[1]) * u[1], gelu_tanh(v[2]) * u[2], gelu_tanh(v[3]) * u[3]);
                     } else {
                         const bf16x4 b = load4(p.bias + n0);
@@ -244,19 +256,24 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
                     }
                 }
             }
-            __syncthreads();
+          }
+          __syncthreads();
+#pragma unroll
+          for (int i = g0; i < (g0 + GROUP < MT ? g0 + GROUP : MT); ++i) {
+            const unsigned char* const tbuf = obuf + (i - g0) * TILE_B;
 #pragma unroll
             for (int ps = 0; ps < 32 / RPP; ++ps) {
                 const int row = ps * RPP + tid / CPR, ch = tid % CPR;
                 const int mm = m0 + i * 32 + row;
                 const int n = nbase + ch * (16 / ESZ);
-                if (mm < p.M && n < ncols) {
-                    const uint4 val = *(const uint4*)(obuf + row * ROWB + ch * 16);
+                if (mm < p.M && n < ncols && !KO(p, 8)) {                        // (KO 8: no global stores)
+                    const uint4 val = *(const uint4*)(tbuf + row * ROWB + ch * 16);
                     if constexpr (EPI == EPI_PARTIAL) *(uint4*)(p.partial + (size_t)split * p.pstride + (size_t)mm * p.ldp + n) = val;
                     else *(uint4*)(p.out + (size_t)mm * p.ldo + n) = val;
                 }
             }
-            __syncthreads();
+          }
+          if (g0 + GROUP < MT) __syncthreads();
         }
         return;
     }
@@ -329,11 +346,37 @@ void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int
     }
 }
 
-template <int WN, int MT, int NT, int EPI>
+// Workgroup -> block tile.  Row blocks come in two sizes when MIXED: the first n_big blocks have MT 32-row tiles, the
+// others MT - 1, so that M rows are covered with ceil(M / 32) tiles instead of a multiple of MT (788 rows: 7 + 6 + 6 + 6 =
+// 25 tiles where four 7-tile blocks would compute 28).
+template <int WN, int MT, int NT, int EPI, bool MIXED>
+__global__ __launch_bounds__(WN * 64, (MT <= 2 && WN == 4 ? 2 : 1))
+void gemm_mfma_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int stages_per_split, int n_big) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int total = m_blocks * n_blocks * p.nsplit;
+    const int lid = xcd_remap(blockIdx.x, total);
+    const int split = lid / (m_blocks * n_blocks);
+    const int rem = lid - split * (m_blocks * n_blocks);
+    const int n_blk = rem / m_blocks;
+    const int m_blk = rem - n_blk * m_blocks;
+    if constexpr (MIXED) {
+        if (m_blk < n_big) gemm_block<WN, MT, NT, EPI>(p, smem_raw, m_blk * (MT * 32), n_blk, split, stages_total, stages_per_split);
+        else gemm_block<WN, MT - 1, NT, EPI>(p, smem_raw, n_big * (MT * 32) + (m_blk - n_big) * ((MT - 1) * 32), n_blk, split, stages_total, stages_per_split);
+    } else {
+        gemm_block<WN, MT, NT, EPI>(p, smem_raw, m_blk * (MT * 32), n_blk, split, stages_total, stages_per_split);
+    }
+}
+
+template <int WN, int MT, int NT, int EPI, bool MIXED>
 int launch_cfg(const GemmP& p, hipStream_t s) {
     constexpr int BM = MT * 32;
     constexpr int HALF = EpiTraits<EPI>::dual ? NT / 2 : NT;
-    const int m_blocks = (p.M + BM - 1) / BM;
+    const int tiles = (p.M + 31) / 32;
+    int m_blocks = (tiles + MT - 1) / MT, n_big = m_blocks;
+    if (MIXED) {
+        n_big = tiles - m_blocks * (MT - 1);               // blocks that need the MT-th tile
+        if (n_big < 0) n_big = 0;
+    }
     const int n_blocks = ((p.N16 + 1) / 2 + WN * HALF - 1) / (WN * HALF);
     const int stages_total = p.K32p / 2;
     const int nsplit = p.nsplit < 1 ? 1 : p.nsplit;
@@ -341,34 +384,38 @@ int launch_cfg(const GemmP& p, hipStream_t s) {
     if ((nsplit - 1) * sps >= stages_total) return 3;      // an empty split would leave its partial unwritten
     if (MT > 4 && ((sps & 1) || (stages_total & 1))) return 3;              // the large tiles consume K stages in pairs
     GemmP q = p; q.nsplit = nsplit;
-    // three K-stage buffers; the row-major epilogues stage one 32-row output tile in the same memory
+#ifdef RTVLA_TUNING
+    q.ko = rtvla_tuning_ko();
+#endif
+    // three K-stage buffers; the row-major epilogues stage 32-row output tiles in the same memory
     const size_t epi_bytes = (size_t)32 * (WN * HALF * 32 * (EPI == EPI_PARTIAL ? 4 : 2) + 16);
     const size_t smem = std::max((size_t)3 * BM * 64 * sizeof(bf16_t), epi_bytes);
-    auto kern = gemm_mfma_kernel<WN, MT, NT, EPI>;
+    auto kern = gemm_mfma_kernel<WN, MT, NT, EPI, MIXED>;
     if (smem > 65536) {
         static bool done = false;
         if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
     }
-    hipLaunchKernelGGL(kern, dim3(m_blocks * n_blocks * nsplit), dim3(WN * 64), smem, s, q, m_blocks, n_blocks, stages_total, sps);
+    hipLaunchKernelGGL(kern, dim3(m_blocks * n_blocks * nsplit), dim3(WN * 64), smem, s, q, m_blocks, n_blocks, stages_total, sps, n_big);
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 
 template <int EPI>
 int launch_epi(const GemmP& p, int tile, hipStream_t s) {
     switch (tile) {
-        case TILE_224x256: return launch_cfg<4, 7, 2, EPI>(p, s);
-        case TILE_160x256: return launch_cfg<4, 5, 2, EPI>(p, s);
-        case TILE_128x256: return launch_cfg<4, 4, 2, EPI>(p, s);
-        case TILE_64x256:  return launch_cfg<4, 2, 2, EPI>(p, s);
-        case TILE_64x128:  if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 2, 1, EPI>(p, s); else return 2;
-        case TILE_128x128: if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 4, 1, EPI>(p, s); else return 2;
+        case TILE_224x256: return launch_cfg<4, 7, 2, EPI, true>(p, s);
+        case TILE_192x256: return launch_cfg<4, 6, 2, EPI, true>(p, s);
+        case TILE_160x256: return launch_cfg<4, 5, 2, EPI, true>(p, s);
+        case TILE_128x256: return launch_cfg<4, 4, 2, EPI, true>(p, s);
+        case TILE_64x256:  return launch_cfg<4, 2, 2, EPI, false>(p, s);
+        case TILE_64x128:  if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 2, 1, EPI, false>(p, s); else return 2;
+        case TILE_128x128: if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 4, 1, EPI, false>(p, s); else return 2;
     }
     return 2;
 }
 
 }  // namespace
 
-int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {224, 160, 128, 64, 64, 128}; return v[tile]; }
+int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {224, 192, 160, 128, 64, 64, 128}; return v[tile]; }
 int gemm_tile_bn(int tile) { return tile >= TILE_64x128 ? 128 : 256; }
 
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {

@@ -58,9 +58,12 @@ struct GemmP {
     float* partial; int ldp; size_t pstride;   // [split][row][ldp]
     const bf16_t* rope;                        // [row][256] = cos0 sin0 cos1 sin1 ...
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt;
+    RTVLA_KO_FIELD
 };
-// workgroup tile (rows x columns), 4 waves each owning 64 columns (two 32-column MFMA tiles)
-enum GemmTile { TILE_224x256 = 0, TILE_160x256, TILE_128x256, TILE_64x256, TILE_64x128, TILE_128x128, TILE_COUNT };
+// workgroup tile (rows x columns), 4 waves each owning 64 columns (two 32-column MFMA tiles).  The tiles of 128 rows and
+// more by 256 columns are upper bounds: their launches mix row blocks of that many and of 32 fewer rows so that the
+// blocks cover ceil(M / 32) 32-row tiles exactly.
+enum GemmTile { TILE_224x256 = 0, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_64x128, TILE_128x128, TILE_COUNT };
 int gemm_tile_bm(int tile);
 int gemm_tile_bn(int tile);
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s);

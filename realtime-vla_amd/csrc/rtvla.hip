@@ -122,7 +122,7 @@ constexpr int64_t ATTN_PARTIAL_FLOATS = 32 * 16 * (16 * 64 * 4 + 32);   // 32 ro
 // their load latency; all workgroups together cannot pull more than ~20 TB/s out of L2; every launch pays a
 // fixed ramp and an epilogue that grows with the tile; split-K adds the reduce pass over the fp32 partials.
 TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what) {
-    static const int tiles[] = {TILE_224x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};
+    static const int tiles[] = {TILE_224x256, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};
     static const int splits[] = {1, 2, 3, 4, 6, 8};
 #ifdef RTVLA_TUNING
     // tuning builds only: force tile / split for the launches whose name contains RTVLA_FORCE_FOR
@@ -140,7 +140,9 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
         if (dual && bn < 256) continue;
         const int bn16 = bn / 16 / (dual ? 2 : 1);
         const int mb = (M + bm - 1) / bm, nb = (ncols16 + bn16 - 1) / bn16;
-        const int mt = bm / 32, nt = bn / 128;
+        const int nt = bn / 128;
+        // the 256-column tiles of 128 rows and more mix row blocks of bm and bm - 32 rows: average 32-row tiles per block
+        const double mt = (bm >= 128 && bn == 256) ? (double)((M + 31) / 32) / mb : bm / 32;
         if (!dual && tile == TILE_64x256) continue;        // measured: 64x128 is never slower than 64x256 for the single-weight GEMMs
         const int occ = bm <= 64 ? 2 : 1;
         for (int sp : splits) {
