@@ -125,6 +125,17 @@ int rtvla_buffer_info(const rtvla_ctx* ctx, int index, const char** name, size_t
  * hipStream_t passed as void*); the caller synchronises. */
 int rtvla_prepare(rtvla_ctx* ctx, void* hip_stream);
 
+/* Saving the re-tiled weights across processes (no reference counterpart; the reference re-reads its checkpoint and
+ * has no derived layout).  After rtvla_prepare the first rtvla_tiled_bytes bytes of the workspace hold every re-tiled
+ * weight and nothing else; they depend only on the weights, the model kind, the layer counts and the tile layout
+ * (rtvla_tile_layout_version, raised whenever that layout changes).  A caller may save that region and, in a later
+ * process with the same weights bound, copy it back to the start of the workspace and call rtvla_prepare_with_tiles
+ * instead of rtvla_prepare: it does everything rtvla_prepare does except the re-tiling. */
+#define RTVLA_TILE_LAYOUT_VERSION 2
+size_t rtvla_tiled_bytes(const rtvla_ctx* ctx);
+int rtvla_tile_layout_version(void);
+int rtvla_prepare_with_tiles(rtvla_ctx* ctx, void* hip_stream);
+
 /* Enqueue one whole forward (pi0_model pi0_infer.py:1232-1236 / pi05_model pi05_infer.py:525-528)
  * on the stream: no allocation, no synchronisation, no host read - capturable.  Inputs are read
  * from the bound io buffers; the result is left in `diffusion_noise`. */

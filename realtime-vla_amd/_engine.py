@@ -1,9 +1,12 @@
 """Shared host logic of Pi0Inference / Pi05Inference: tensor ownership (PyTorch-ROCm), binding
 to the C ABI, RoPE tables, graph capture.  PyTorch is used only to own device memory and for
 the input staging copies; every kernel of the forward lives in librtvla.so."""
+import os
+
 import torch
 
 import rtvla_capi as capi
+from tile_cache import TileCache, fingerprint
 
 _DTYPES = {2: torch.bfloat16, 4: torch.int32}
 
@@ -20,7 +23,7 @@ def rope_table(start, count, device):
 
 
 class Engine:
-    def __init__(self, model, checkpoint, num_views, prompt_len, chunk_size, num_steps=10, skip_keys=()):
+    def __init__(self, model, checkpoint, num_views, prompt_len, chunk_size, num_steps=10, skip_keys=(), tile_cache=None):
         if not torch.cuda.is_available():
             raise RuntimeError("realtime-vla_amd needs a ROCm GPU (MI355X / gfx950); there is no CPU path")
         self.device = torch.device("cuda", torch.cuda.current_device())
@@ -29,6 +32,9 @@ class Engine:
             vision_layers = int(checkpoint["vision_attn_qkv_w"].shape[0])
         if "encoder_attn_qkv_w" in checkpoint:
             llm_layers = int(checkpoint["encoder_attn_qkv_w"].shape[0])
+        self.model, self.vision_layers, self.llm_layers = model, vision_layers, llm_layers
+        self.tile_cache = TileCache(tile_cache) if isinstance(tile_cache, (str, os.PathLike)) else tile_cache
+        self.tile_cache_hit = None                                   # True / False after prepare() when a cache is in use
         self.ctx = capi.Context(model, num_views, prompt_len, chunk_size, num_steps, vision_layers, llm_layers)
         self.weights, self.buffers = {}, {}
         for name, elem, shape, is_weight, required in self.ctx.tensors():
@@ -54,16 +60,31 @@ class Engine:
         self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
         self.ctx.bind_workspace(self.workspace.data_ptr(), nbytes)
         # views of the library's internal activations, under the reference's buffer names where one exists
+        self.tiled_sources = {"decoder_action_fused_out_proj_w", "decoder_action_out_proj_w", "decoder_action_out_proj_b"}
         for name, off, rows, cols, ld, elem in self.ctx.buffers():
             if name.startswith("t_"):
+                self.tiled_sources.add(name[2:])                     # the weight this re-tiled copy is made from
                 continue
             flat = self.workspace[off:off + rows * ld * elem].view(torch.bfloat16 if elem == 2 else torch.float32)
             self.buffers.setdefault(name, flat.view(rows, ld)[:, :cols])
         self.stream = torch.cuda.current_stream(self.device)
 
     def prepare(self):
-        self.ctx.prepare(self.stream.cuda_stream)
+        """rtvla_prepare; with a tile cache the re-tiled weights come from its file when one matches this checkpoint
+        (fingerprint of the weights as they sit on the device), and are saved there after the first re-tiling."""
+        if self.tile_cache is None:
+            self.ctx.prepare(self.stream.cuda_stream)
+            torch.cuda.synchronize(self.device)
+            return
+        lib = capi.load()
+        ident = (lib.rtvla_tile_layout_version(), self.model, self.vision_layers, self.llm_layers)
+        key = fingerprint({k: v for k, v in self.weights.items() if k in self.tiled_sources})
+        region = self.workspace[: self.ctx.tiled_bytes()]
+        self.tile_cache_hit = self.tile_cache.load_into(key, *ident, region)
+        self.ctx.prepare(self.stream.cuda_stream, tiles_loaded=self.tile_cache_hit)
         torch.cuda.synchronize(self.device)
+        if not self.tile_cache_hit:
+            self.tile_cache.store(key, *ident, region)
 
     def capture(self):
         """One eager forward, then capture into a HIP graph on a side stream

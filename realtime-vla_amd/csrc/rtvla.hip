@@ -523,11 +523,13 @@ struct Sched {
         }
     }
 
-    // one-time device work
-    void prepare() {
+    // one-time device work.  With `tiles_loaded` the re-tiled weights (the first rtvla_tiled_bytes of the workspace) were
+    // filled in by the caller from a copy saved after an earlier prepare, and only the rest is done.
+    void prepare(bool tiles_loaded) {
         const int V = d.vision_layers, L = d.llm_layers;
         launch_fill_zero(c->ws + c->act_begin, c->ws_bytes - c->act_begin, s);
         auto tile = [&](const char* src, const char* dst, int K, int N, int layers) {
+            if (tiles_loaded) return;
             for (int i = 0; i < layers; ++i) launch_pretile(c->W(src, (size_t)K * N, i), K, N, c->TW(dst, i), c->tgroup.at(dst), c->twide.at(dst), s);
         };
         tile("vision_patch_embedding_w", "t_vision_patch_embedding_w", 588, 1152, 1);
@@ -553,11 +555,13 @@ struct Sched {
         }
         // Pi05: out-proj scaled by -1/num_steps (pi05_infer.py:669-671), then the time conditioning (:673-722)
         const float dt = -1.0f / (float)d.num_steps;
-        launch_copy_bytes(c->W("decoder_action_out_proj_w"), c->B("decoder_out_proj_w_scaled"), 1024 * 32 * 2, s);
-        launch_scale_inplace(c->B("decoder_out_proj_w_scaled"), 1024 * 32, dt, s);
-        launch_copy_bytes(c->W("decoder_action_out_proj_b"), c->B("decoder_out_proj_b_scaled"), 64, s);
-        launch_scale_inplace(c->B("decoder_out_proj_b_scaled"), 32, dt, s);
-        launch_pretile(c->B("decoder_out_proj_w_scaled"), 1024, 32, c->TW("t_decoder_out_proj_w"), 1, 0, s);
+        if (!tiles_loaded) {                               // (the scaled copies sit in the saved region as well)
+            launch_copy_bytes(c->W("decoder_action_out_proj_w"), c->B("decoder_out_proj_w_scaled"), 1024 * 32 * 2, s);
+            launch_scale_inplace(c->B("decoder_out_proj_w_scaled"), 1024 * 32, dt, s);
+            launch_copy_bytes(c->W("decoder_action_out_proj_b"), c->B("decoder_out_proj_b_scaled"), 64, s);
+            launch_scale_inplace(c->B("decoder_out_proj_b_scaled"), 32, dt, s);
+            launch_pretile(c->B("decoder_out_proj_w_scaled"), 1024, 32, c->TW("t_decoder_out_proj_w"), 1, 0, s);
+        }
         tile("decoder_time_mlp_in_w", "t_decoder_time_mlp_in_w", 1024, 1024, 1);
         tile("decoder_time_mlp_out_w", "t_decoder_time_mlp_out_w", 1024, 1024, 1);
         tile("decoder_pre_attn_norm_mod_w", "t_decoder_pre_attn_norm_mod_w", 1024, 3072, L);
@@ -695,16 +699,21 @@ int rtvla_buffer_info(const rtvla_ctx* c, int index, const char** name, size_t* 
     return RTVLA_OK;
 }
 
-int rtvla_prepare(rtvla_ctx* c, void* stream) {
+static int prepare_impl(rtvla_ctx* c, void* stream, bool tiles_loaded) {
     if (int rc = check_ready(c, false)) return rc;
     c->status = 0; c->launches = 0; c->kernels = 0;
-    Sched(c, (hipStream_t)stream).prepare();
+    Sched(c, (hipStream_t)stream).prepare(tiles_loaded);
     if (c->status) return c->status;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(c, e, "prepare");
     c->prepared = true;
     return RTVLA_OK;
 }
+
+int rtvla_prepare(rtvla_ctx* c, void* stream) { return prepare_impl(c, stream, false); }
+int rtvla_prepare_with_tiles(rtvla_ctx* c, void* stream) { return prepare_impl(c, stream, true); }
+size_t rtvla_tiled_bytes(const rtvla_ctx* c) { return c ? c->act_begin : 0; }
+int rtvla_tile_layout_version(void) { return RTVLA_TILE_LAYOUT_VERSION; }
 
 int rtvla_forward(rtvla_ctx* c, void* stream) {
     if (int rc = check_ready(c, true)) return rc;

@@ -19,6 +19,7 @@ class Pi05Inference:
         discrete_state_input: bool = True,
         max_prompt_text: str | None = None,
         state_dim_for_max_prompt: int | None = None,
+        tile_cache=None,                 # not in the reference: directory that keeps the re-tiled weights across processes
     ):
         self.discrete_state_input = discrete_state_input
         self.tokenizer_path = tokenizer_path
@@ -55,7 +56,8 @@ class Pi05Inference:
         # (the reference does both on the host per call, pi05_infer.py:769-785, :811-822).
         self.device_prompt = "embedding_weight" in checkpoint and (discrete_state_input or 'language_embeds' not in checkpoint)
         self._engine = Engine(capi.PI05, checkpoint, num_views, self.max_prompt_len, chunk_size,
-                              skip_keys=("language_embeds",) if self.device_prompt else ("embedding_weight", "language_embeds"))
+                              skip_keys=("language_embeds",) if self.device_prompt else ("embedding_weight", "language_embeds"),
+                              tile_cache=tile_cache)
         self.weights = self._engine.weights
         self.buffers = self._engine.buffers
         dev = self._engine.device

@@ -7,12 +7,13 @@ from _engine import Engine, rope_table
 
 
 class Pi0Inference:
-    def __init__(self, checkpoint, num_views, chunk_size):
+    def __init__(self, checkpoint, num_views, chunk_size, tile_cache=None):
+        """`tile_cache` (not in the reference): a directory in which the re-tiled weights are kept across processes."""
         self.num_views = num_views
         self.chunk_size = chunk_size
         encoded_prompt = checkpoint['language_embeds']          # KeyError if absent, as in the reference
         self.prompt_len = len(encoded_prompt)
-        self._engine = Engine(capi.PI0, checkpoint, num_views, self.prompt_len, chunk_size)
+        self._engine = Engine(capi.PI0, checkpoint, num_views, self.prompt_len, chunk_size, tile_cache=tile_cache)
         self.weights = self._engine.weights
         self.buffers = self._engine.buffers
 

@@ -50,6 +50,9 @@ SYMBOLS = {
                                          ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
                                          ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32)]),
     "rtvla_prepare": (ctypes.c_int, [_P, _P]),
+    "rtvla_prepare_with_tiles": (ctypes.c_int, [_P, _P]),
+    "rtvla_tiled_bytes": (ctypes.c_size_t, [_P]),
+    "rtvla_tile_layout_version": (ctypes.c_int, []),
     "rtvla_forward": (ctypes.c_int, [_P, _P]),
     "rtvla_forward_stage": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "rtvla_graph_capture": (ctypes.c_int, [_P, _P]),
@@ -150,8 +153,12 @@ class Context:
     def bind_workspace(self, ptr, nbytes):
         self.check(self.lib.rtvla_bind_workspace(self.handle, _P(ptr), nbytes))
 
-    def prepare(self, stream):
-        self.check(self.lib.rtvla_prepare(self.handle, _P(stream)))
+    def prepare(self, stream, tiles_loaded=False):
+        fn = self.lib.rtvla_prepare_with_tiles if tiles_loaded else self.lib.rtvla_prepare
+        self.check(fn(self.handle, _P(stream)))
+
+    def tiled_bytes(self):
+        return self.lib.rtvla_tiled_bytes(self.handle)
 
     def forward(self, stream):
         self.check(self.lib.rtvla_forward(self.handle, _P(stream)))

@@ -53,3 +53,38 @@ def test_safetensors_round_trip(tmp_path):
     assert set(got) == set(ck)
     for k in ck:
         assert got[k].dtype == ck[k].dtype and torch.equal(got[k], ck[k])
+
+
+def test_weight_fingerprint_is_exact_and_order_sensitive():
+    import tile_cache as tc
+    ck = _small_checkpoint()
+    a = tc.fingerprint(ck)
+    assert a == tc.fingerprint({k: v.clone() for k, v in reversed(list(ck.items()))}) and len(a) == 32
+    flipped = {k: v.clone() for k, v in ck.items()}
+    flipped["vision_attn_qkv_b"][0, 5] += 1.0
+    assert tc.fingerprint(flipped) != a
+    swapped = {k: v.clone() for k, v in ck.items()}
+    w = swapped["vision_attn_qkv_b"]
+    w[0, 1], w[0, 2] = ck["vision_attn_qkv_b"][0, 2], ck["vision_attn_qkv_b"][0, 1]      # same multiset of values, other order
+    assert not torch.equal(w, ck["vision_attn_qkv_b"]) and tc.fingerprint(swapped) != a
+    renamed = dict(ck); renamed["other_name"] = renamed.pop("language_embeds")
+    assert tc.fingerprint(renamed) != a
+
+
+def test_tile_cache_file_round_trip_and_header_checks(tmp_path):
+    import tile_cache as tc
+    cache = tc.TileCache(tmp_path / "tiles")
+    key = bytes(range(32))
+    region = torch.arange(5000, dtype=torch.int64).to(torch.uint8)
+    assert not cache.load_into(key, 2, 0, 27, 18, torch.empty_like(region))               # nothing stored yet
+    path = cache.store(key, 2, 0, 27, 18, region)
+    assert os.path.getsize(path) == 64 + 5000
+    back = torch.zeros_like(region)
+    assert cache.load_into(key, 2, 0, 27, 18, back) and torch.equal(back, region)
+    for other in ((3, 0, 27, 18), (2, 1, 27, 18), (2, 0, 2, 18), (2, 0, 27, 2)):           # layout version, model, layer counts
+        assert not cache.load_into(key, *other, torch.zeros_like(region))
+    assert not cache.load_into(key, 2, 0, 27, 18, torch.zeros(4999, dtype=torch.uint8))  # another size
+    assert not cache.load_into(bytes(32), 2, 0, 27, 18, torch.zeros_like(region))         # another checkpoint
+    with open(path, "r+b") as f:                                                           # a truncated / foreign file
+        f.write(b"garbage!")
+    assert not cache.load_into(key, 2, 0, 27, 18, torch.zeros_like(region))

@@ -381,3 +381,32 @@ def test_constructor_errors_match_the_reference():
     m = Pi0Inference(ck, 1, 10)
     with pytest.raises(RuntimeError):
         m.forward(torch.zeros(2, 224, 224, 3), torch.zeros(32), torch.zeros(10, 32))
+
+
+def test_start_from_the_tile_cache_gives_bit_identical_actions(tmp_path):
+    """Second construction on the same checkpoint loads the re-tiled weights from the cache file instead of
+    re-tiling; a changed weight misses the cache."""
+    from pi0_infer import Pi0Inference
+    from pi05_infer import Pi05Inference
+    ck = syn.pi0_checkpoint(41, 3, "cuda:0", 2, 2, norms="random")
+    img, state, noise = syn.observation(41, 1, 9, "cuda:0")
+    plain = Pi0Inference(ck, 1, 9).forward(img, state, noise).clone()
+    first = Pi0Inference(ck, 1, 9, tile_cache=tmp_path)
+    assert first._engine.tile_cache_hit is False and len(list(tmp_path.iterdir())) == 1
+    second = Pi0Inference(ck, 1, 9, tile_cache=str(tmp_path))
+    assert second._engine.tile_cache_hit is True
+    assert torch.equal(first.forward(img, state, noise), plain) and torch.equal(second.forward(img, state, noise), plain)
+    # another prompt re-uses the tiles (the prompt is not re-tiled), another weight does not
+    ck2 = dict(ck, language_embeds=syn.language_embeds(42, 5, "cuda:0"))
+    assert Pi0Inference(ck2, 1, 9, tile_cache=tmp_path)._engine.tile_cache_hit is True
+    ck3 = dict(ck); ck3["decoder_ffn_up_w"] = ck["decoder_ffn_up_w"].clone(); ck3["decoder_ffn_up_w"][1, 7, 9] += 0.5
+    third = Pi0Inference(ck3, 1, 9, tile_cache=tmp_path)
+    assert third._engine.tile_cache_hit is False and len(list(tmp_path.iterdir())) == 2
+    assert not torch.equal(third.forward(img, state, noise), plain)
+    # Pi05: the scaled output projection and the conditioning are rebuilt around the cached tiles
+    ck5 = syn.pi05_checkpoint(43, 4, "cuda:0", 1, 2, state_tokens=2, norms="random")
+    img5, _, noise5 = syn.observation(43, 1, 6, "cuda:0")
+    a = Pi05Inference(ck5, 1, 6, discrete_state_input=False, tile_cache=tmp_path)
+    b = Pi05Inference(ck5, 1, 6, discrete_state_input=False, tile_cache=tmp_path)
+    assert (a._engine.tile_cache_hit, b._engine.tile_cache_hit) == (False, True)
+    assert torch.equal(a.forward(img5, noise5), b.forward(img5, noise5))
