@@ -196,6 +196,10 @@ size_t rtvla_linear_workspace_bytes(int M, int K, int N, int tile, int nsplit);
 int rtvla_linear(const void* x, int M, int K, const void* w, int N, const void* bias, void* out, void* workspace,
                  size_t workspace_bytes, int tile, int nsplit, void* hip_stream);
 int rtvla_linear_tile_shape(int tile, int* rows, int* cols);
+/* Measurement helper: as rtvla_linear without bias, then the compute launches alone (GEMM, and reduce when split)
+ * `iters` times in a temporary graph on `hip_stream` (not the null stream), mean milliseconds of one. */
+int rtvla_time_linear(const void* x, int M, int K, const void* w, int N, void* out, void* workspace, size_t workspace_bytes,
+                      int tile, int nsplit, int iters, void* hip_stream, float* mean_ms);
 
 /* ---- observation pre-/post-processing either side of the forward (context-free, capturable) ----------------
  * The reference does these on the host per observation (test.py:88-201).  All pointers are device pointers. */

@@ -893,56 +893,84 @@ size_t rtvla_linear_workspace_bytes(int M, int K, int N, int tile, int nsplit) {
     return plan_linear(M, K, N, tile, nsplit, &pl) == RTVLA_OK ? pl.total : 0;
 }
 
-int rtvla_linear(const void* x, int M, int K, const void* w, int N, const void* bias, void* out, void* workspace, size_t workspace_bytes,
-                 int tile, int nsplit, void* stream) {
+static int linear_impl(const void* x, int M, int K, const void* w, int N, const void* bias, void* out, void* workspace, size_t workspace_bytes,
+                       int tile, int nsplit, hipStream_t s, int timed_iters, float* mean_ms) {
     if (!x || !w || !out || !workspace || ((uintptr_t)workspace & 255)) return RTVLA_ERR_ARG;
     LinearPlan pl;
     if (int rc = plan_linear(M, K, N, tile, nsplit, &pl)) return rc;
     if (workspace_bytes < pl.total) return RTVLA_ERR_SIZE;
-    hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
     bf16_t* zbias = (bf16_t*)(ws + pl.bias_off);
     launch_fill_zero(zbias, ((size_t)N * 2 + 255) & ~(size_t)255, s);
     const bf16_t* b = bias ? (const bf16_t*)bias : zbias;
-    int rc = 0;
-    if (pl.skinny) {
-        bf16_t* wt = (bf16_t*)(ws + pl.w_off);
-        launch_pretile((const bf16_t*)w, K, N, wt, 1, 0, s);
-        SkinnyP p{};
-        p.A = (const bf16_t*)x; p.lda = K; p.M = M; p.B0 = wt; p.K = K; p.N16 = n16_tiles(N); p.K32p = k32_padded(K);
-        p.norm = SN_NONE; p.eps = 1e-6f; p.out = (bf16_t*)out; p.ldo = N; p.bias = b;
-        if (K == 1024) rc = launch_skinny(p, SK_BIAS, s);
-        else {
-            // the K = 2048 / 4096 variants exist with the residual epilogue only (O and down projections): out = 0 + acc + bias
-            launch_fill_zero(out, (size_t)M * N * 2, s);
-            rc = launch_skinny(p, SK_RES, s);
-        }
-    } else {
-        bf16_t* a = (bf16_t*)(ws + pl.a_off);
-        bf16_t* wt = (bf16_t*)(ws + pl.w_off);
+    bf16_t* a = (bf16_t*)(ws + pl.a_off);
+    bf16_t* wt = (bf16_t*)(ws + pl.w_off);
+    // operands into the layouts the kernels read
+    if (pl.skinny) launch_pretile((const bf16_t*)w, K, N, wt, 1, 0, s);
+    else {
         launch_fill_zero(a, ((size_t)M * pl.K128 * 2 + 255) & ~(size_t)255, s);       // K is zero-padded to the 128-wide stage pair
         launch_copy_rows((const bf16_t*)x, K, a, pl.K128, M, K, s);
         launch_pretile((const bf16_t*)w, K, N, wt, 8, 1, s);
+    }
+    auto compute = [&]() -> int {
+        if (pl.skinny) {
+            SkinnyP p{};
+            p.A = (const bf16_t*)x; p.lda = K; p.M = M; p.B0 = wt; p.K = K; p.N16 = n16_tiles(N); p.K32p = k32_padded(K);
+            p.norm = SN_NONE; p.eps = 1e-6f; p.out = (bf16_t*)out; p.ldo = N; p.bias = b;
+            if (K == 1024) return launch_skinny(p, SK_BIAS, s);
+            // the K = 2048 / 4096 variants exist with the residual epilogue only (O and down projections): out = 0 + acc + bias
+            launch_fill_zero(out, (size_t)M * N * 2, s);
+            return launch_skinny(p, SK_RES, s);
+        }
         GemmP p{};
         p.A = a; p.lda = pl.K128; p.a_rows = M; p.M = M; p.B0 = wt; p.bgroup = 8;
         p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.nsplit = pl.nsplit;
-        if (pl.partial) {
-            float* part = (float*)(ws + pl.part_off);
-            p.partial = part; p.ldp = N; p.pstride = (size_t)M * N;
-            rc = launch_gemm(p, EPI_PARTIAL, pl.tile, s);
-            if (!rc) {
-                ReduceP r{};
-                r.partial = part; r.pstride = p.pstride; r.ldp = N; r.nsplit = pl.nsplit; r.bias = b;
-                r.x = (bf16_t*)out; r.ldx = N; r.M = M; r.N = N; r.norm = NORM_NONE;
-                rc = launch_reduce(r, s);
-            }
-        } else {
+        if (!pl.partial) {
             p.out = (bf16_t*)out; p.ldo = N; p.bias = b;
-            rc = launch_gemm(p, EPI_BIAS, pl.tile, s);
+            return launch_gemm(p, EPI_BIAS, pl.tile, s);
         }
-    }
+        float* part = (float*)(ws + pl.part_off);
+        p.partial = part; p.ldp = N; p.pstride = (size_t)M * N;
+        if (int rc = launch_gemm(p, EPI_PARTIAL, pl.tile, s)) return rc;
+        ReduceP r{};
+        r.partial = part; r.pstride = p.pstride; r.ldp = N; r.nsplit = pl.nsplit; r.bias = b;
+        r.x = (bf16_t*)out; r.ldx = N; r.M = M; r.N = N; r.norm = NORM_NONE;
+        return launch_reduce(r, s);
+    };
+    int rc = compute();
     if (rc) return rc == 3 ? RTVLA_ERR_LIMIT : RTVLA_ERR_DEVICE;      // 3: this tile cannot take this K / split
-    return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
+    if (hipGetLastError() != hipSuccess) return RTVLA_ERR_DEVICE;
+    if (timed_iters <= 0) return RTVLA_OK;
+    // measurement: the compute launches alone, `timed_iters` times in a temporary graph, one untimed and one timed replay
+    if (hipStreamSynchronize(s) != hipSuccess) return RTVLA_ERR_DEVICE;
+    hipGraph_t g = nullptr; hipGraphExec_t ge = nullptr; hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) return RTVLA_ERR_DEVICE;
+    for (int i = 0; i < timed_iters && !rc; ++i) rc = compute();
+    if (hipStreamEndCapture(s, &g) != hipSuccess || rc) rc = RTVLA_ERR_DEVICE;
+    if (!rc && hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) != hipSuccess) rc = RTVLA_ERR_DEVICE;
+    if (!rc && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) rc = RTVLA_ERR_DEVICE;
+    if (!rc) {
+        hipGraphLaunch(ge, s);
+        hipEventRecord(e0, s); hipGraphLaunch(ge, s); hipEventRecord(e1, s);
+        if (hipEventSynchronize(e1) != hipSuccess) rc = RTVLA_ERR_DEVICE;
+        else { float ms = 0.f; hipEventElapsedTime(&ms, e0, e1); *mean_ms = ms / timed_iters; }
+    }
+    if (e0) hipEventDestroy(e0);
+    if (e1) hipEventDestroy(e1);
+    if (ge) hipGraphExecDestroy(ge);
+    if (g) hipGraphDestroy(g);
+    return rc;
+}
+
+int rtvla_linear(const void* x, int M, int K, const void* w, int N, const void* bias, void* out, void* workspace, size_t workspace_bytes,
+                 int tile, int nsplit, void* stream) {
+    return linear_impl(x, M, K, w, N, bias, out, workspace, workspace_bytes, tile, nsplit, (hipStream_t)stream, 0, nullptr);
+}
+
+int rtvla_time_linear(const void* x, int M, int K, const void* w, int N, void* out, void* workspace, size_t workspace_bytes,
+                      int tile, int nsplit, int iters, void* stream, float* mean_ms) {
+    if (iters < 1 || !mean_ms || !stream) return RTVLA_ERR_ARG;      // (a graph cannot be captured on the null stream)
+    return linear_impl(x, M, K, w, N, nullptr, out, workspace, workspace_bytes, tile, nsplit, (hipStream_t)stream, iters, mean_ms);
 }
 
 int rtvla_linear_tile_shape(int tile, int* rows, int* cols) {

@@ -66,6 +66,8 @@ SYMBOLS = {
     "rtvla_pretile": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P]),
     "rtvla_linear_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 5),
     "rtvla_linear": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, ctypes.c_int, _P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, _P]),
+    "rtvla_time_linear": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, ctypes.c_int, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                                         ctypes.c_int, _P, ctypes.POINTER(ctypes.c_float)]),
     "rtvla_linear_tile_shape": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
     "rtvla_preprocess_image_scratch": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "rtvla_preprocess_image": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P, ctypes.c_size_t, _P]),
