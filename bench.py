@@ -29,6 +29,7 @@ MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 COPY_PROBE_BYTES = 256 << 20   # size of the calibration copy of --traffic-probe
 PROFILES = os.path.join(ROOT, "profiles")
+PROFILE_TAGS = {"headline": "pi0_3view_p20_c50"}      # workloads that have counter summaries under profiles/
 
 
 def profiled_traffic(file_name, kernel_desc, workload, lib_version):
@@ -120,6 +121,11 @@ def main():
     ap.add_argument("--cpu-runs", type=int, default=3, help="timed CPU-oracle forwards after one warm-up (median reported)")
     ap.add_argument("--transforms", action="store_true",
                     help="measure the observation pre-/post-processing kernels (3 camera frames of 480x640, state, actions) instead of the forward")
+    ap.add_argument("--launch-times", action="store_true",
+                    help="print the mean duration of every kernel launch of one SigLIP, prefix and action-expert layer (weights cache-warm "
+                         "and cold), measured in temporary graphs, and exit.  With a tuning build of the library (build.py -DRTVLA_TUNING, "
+                         "selected by RTVLA_LIBRARY) --knockouts repeats the action-expert timings with parts of the kernels switched off")
+    ap.add_argument("--knockouts", default="", help="comma-separated RTVLA_KO masks for --launch-times (tuning builds only)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: launch the roofline kernel a few times, then a "
                          "plain 256 MiB device copy whose counter reading calibrates the unit, and exit")
@@ -155,6 +161,31 @@ def main():
     lib_version = capi.load().rtvla_version()
     # index of the gate/up GEMM among the launches of one prefix layer, found by its name
     GEGLU_LAUNCH = next(i for i in range(16) if (ctx.time_launch(capi.STAGE_PREFIX_LAYER, 0, 0, i, 1, stream) or (0, "prefix geglu"))[1].startswith("prefix geglu"))
+    if args.launch_times:
+        for i in range(3):
+            run(noise)
+        torch.cuda.synchronize()
+        rows = []
+        for label, stage in (("siglip", capi.STAGE_VISION_LAYER), ("prefix", capi.STAGE_PREFIX_LAYER), ("action", capi.STAGE_SUFFIX_LAYER)):
+            for idx in range(16):
+                r = ctx.time_launch(stage, 3, 0, idx, 50, stream)
+                if r is None:
+                    break
+                rows.append({"layer": label, "launch": r[1], "warm_us": round(r[0] * 1e3, 2),
+                             "cold_us": round(ctx.time_launch(stage, -1, 0, idx, 3, stream)[0] * 1e3, 2)})
+            rows.append({"layer": label, "launch": "whole layer", "warm_us": round(ctx.time_stage(stage, 3, 0, 50, stream) * 1e3, 2),
+                         "cold_us": round(ctx.time_stage(stage, -1, 0, 3, stream) * 1e3, 2)})
+        out = {"workload": desc, "rtvla_version": lib_version, "launches": rows}
+        if args.knockouts:
+            out["knockouts"] = []
+            for ko in args.knockouts.split(","):
+                os.environ["RTVLA_KO"] = ko
+                out["knockouts"].append({"mask": int(ko), "action_layer_launches_warm_us": {
+                    ctx.time_launch(capi.STAGE_SUFFIX_LAYER, 3, 0, idx, 100, stream)[1]: round(ctx.time_launch(capi.STAGE_SUFFIX_LAYER, 3, 0, idx, 100, stream)[0] * 1e3, 2)
+                    for idx in range(5)}})
+            os.environ["RTVLA_KO"] = "0"
+        print(json.dumps(out))
+        return
     if args.traffic_probe:
         ms, name = ctx.time_launch(capi.STAGE_PREFIX_LAYER, 3, 0, GEGLU_LAUNCH, 5, stream)
         ctx.time_stage(capi.STAGE_SUFFIX_LAYER, -1, 0, 2, stream)          # every action-expert layer, weights cold
@@ -203,7 +234,7 @@ def main():
                 "launch_ms": round(geglu_ms, 4), "launch_ms_cache_warm": round(geglu_warm_ms, 4),
                 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each calibrated on a 256 MiB copy, as recorded in
                 # profiles/ for exactly this kernel variant and library version (null otherwise)
-                "traffic": profiled_traffic("gemm_geglu_hbm_traffic.md", geglu_name, args.config, lib_version),
+                "traffic": profiled_traffic("gemm_geglu_%s_hbm_traffic.md" % PROFILE_TAGS.get(args.config), geglu_name, args.config, lib_version),
                 "kernel_variant": geglu_name,
                 "algorithmic_bytes": 2.0 * (S_e * 2048 + 2 * 2048 * 16384 + S_e * 16384)}
     # the action-expert side: one suffix layer (5 launches) streams 18 D_L-sized weight sets per step
@@ -216,7 +247,7 @@ def main():
                     "achieved": round(hbm, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hbm / HBM_PEAK_GBS, 4),
                     "launch_ms": round(layer_ms, 4), "launch_ms_cache_warm": round(layer_warm_ms, 4),
                     # HBM bytes per layer from rocprofv3 FETCH_SIZE + WRITE_SIZE summed over the layer's kernels (profiles/)
-                    "traffic": profiled_traffic("action_expert_layer_hbm_traffic.md", "action-expert layer", args.config, lib_version),
+                    "traffic": profiled_traffic("action_expert_layer_%s_hbm_traffic.md" % PROFILE_TAGS.get(args.config), "action-expert layer", args.config, lib_version),
                     "algorithmic_bytes": layer_bytes}
     # whole-forward roofline fraction: (F_vis + F_pre) / P_mfma + B_dec / BW  over the measured p50
     v_l = 1152 * 3456 + 1152 * 1152 + 2 * 1152 * 4304
