@@ -262,6 +262,49 @@ def pi05_checkpoint(seed, prompt_len, device="cpu", vision_layers=27, llm_layers
     return ck
 
 
+DM0_VOCAB = 152701
+
+
+def dm0_checkpoint(seed, device="cpu", vision_layers=23, llm_layers=28, std=0.02, vocab=DM0_VOCAB):
+    """Synthetic DM0 checkpoint (keys/shapes of /root/reference/dm0_infer.py:991-1035).  Matrices N(0, std^2); the folded
+    LayerNorm column sums are the column sums of the folded weights, as the converter computes them; norm weights
+    1 + N(0, 0.1^2); `vocab` rows of token embeddings (the reference table has 152701)."""
+    V, L = vision_layers, llm_layers
+    shapes = {
+        "decoder_attn_qkv_w": (L, 1024, 4096), "decoder_attn_o_w": (L, 2048, 1024),
+        "decoder_ffn_gate_w": (L, 1024, 1536), "decoder_ffn_up_w": (L, 1024, 1536), "decoder_ffn_down_w": (L, 1536, 1024),
+        "decoder_action_fused_in_proj_w": (32, 1024), "decoder_action_fused_time_biases": (10, 1024),
+        "decoder_action_mlp_w": (1024, 1024), "decoder_action_mlp_b": (1024,),
+        "decoder_action_fused_out_proj_w": (1024, 32), "decoder_action_fused_out_proj_b": (32,),
+        "llm_attn_qkv_w": (L, 2048, 4096), "llm_attn_o_w": (L, 2048, 2048),
+        "llm_ffn_gate_w": (L, 2048, 6144), "llm_ffn_up_w": (L, 2048, 6144), "llm_ffn_down_w": (L, 6144, 2048),
+        "vision_conv1_w_t": (588, 1024), "vision_class_embedding": (1024,), "vision_pos_emb": (2705, 1024),
+        "vision_fused_qkv_w": (V, 1024, 3072), "vision_out_proj_w": (V, 1024, 1024), "vision_out_proj_b": (V, 1024),
+        "vision_fused_fc_w": (V, 1024, 4096), "vision_proj_w": (V, 4096, 1024), "vision_proj_b": (V, 1024),
+        "vision_ds1_w": (3, 3, 1024, 2048), "vision_ds1_b": (2048,), "vision_ds2_w": (3, 3, 2048, 4096), "vision_ds2_b": (4096,),
+        "vision_projector_w_t": (4096, 2048), "vision_embed_tokens_w": (vocab, 2048),
+    }
+    ck = {k: normal_bf16(seed, k, s, std, device) for k, s in shapes.items()}
+    for k in ("decoder_action_fused_out_proj_w", "decoder_action_fused_out_proj_b"):      # dt = -0.1 folded in, as for Pi0
+        ck[k] = (ck[k].float() * -0.1).to(torch.bfloat16)
+    for k, shape in (("decoder_q_norm_w", (L, 128)), ("decoder_k_norm_w", (L, 128)), ("llm_q_norm_w", (L, 128)), ("llm_k_norm_w", (L, 128)),
+                     ("vision_ln_pre_w", (1024,))):
+        ck[k] = (1.0 + normal_bf16(seed, k, shape, 0.1, device).float()).to(torch.bfloat16)
+    ck["vision_ln_pre_b"] = normal_bf16(seed, "vision_ln_pre_b", (1024,), 0.1, device)
+    for name, n in (("qkv", 3072), ("fc", 4096)):                                           # fp32 tensors of the folded LayerNorm
+        ck["vision_fused_%s_b" % name] = normal_bf16(seed, "vision_fused_%s_b" % name, (V, n), 0.05, device).float()
+        ck["vision_%s_col_sum" % name] = ck["vision_fused_%s_w" % name].float().sum(dim=1)
+    return ck
+
+
+def dm0_observation(seed, num_images, device="cpu", max_lang_len=100, vocab=DM0_VOCAB, draw=0):
+    """Seeded DM0 inputs: images [n,3,728,728] uniform[-1,1) bf16, `max_lang_len` token ids, noise [50,32] ~N(0,1) bf16."""
+    images = uniform_pm1_bf16(seed, "images", (num_images, 3, 728, 728), device)
+    ids = randint(seed, "input_ids", max_lang_len, vocab, device)
+    noise = normal_bf16(seed, "diffusion_noise/%d" % draw, (50, 32), 1.0, device)
+    return images, ids, noise
+
+
 def observation(seed, num_views, chunk_size, device="cpu", draw=0):
     """Seeded inputs: images [v,224,224,3] uniform[-1,1), state [32] and noise [chunk,32] ~N(0,1), bf16.
     `draw` selects an independent noise stream (fresh noise per iteration)."""
