@@ -1,10 +1,13 @@
 // Softmax attention on MFMA, flash style (online softmax, logits never leave registers).
 //
-//  * mqa_kernel    - Gemma multi-query attention, 8 query heads sharing one 256-wide K/V head: the
-//                    prefix pass (/root/reference/pi0_infer.py:819-824, pi05_infer.py:335-360) and
-//                    the action-expert suffix pass with its masks (pi0_infer.py:1041-1120,
-//                    pi05_infer.py:382-478).  Query rows are token*8 + head, so the whole thing is
-//                    a [rows x 256] x [keys x 256]^T problem against one shared K and V.
+//  * mqa_kernel    - attention of G query heads that share one K/V head of width HD, query rows = token*G + head,
+//                    i.e. a [rows x HD] x [keys x HD]^T problem against one shared K and V, optionally batched
+//                    over independent K/V heads (blockIdx.y).  G = 8, HD = 256: Gemma multi-query attention, the
+//                    prefix pass (/root/reference/pi0_infer.py:819-824, pi05_infer.py:335-360) and the
+//                    action-expert suffix pass with its masks (pi0_infer.py:1041-1120, pi05_infer.py:382-478).
+//                    G = 2, HD = 128, 8 K/V heads: DM0's grouped-query attention, causal in the prefix
+//                    (/root/reference/dm0_infer.py:913-918) and unmasked in the action expert (:822-826).
+//                    G = 1, HD = 64, one K/V head per (image, head): DM0's ViT attention (:589-598).
 //  * vision_kernel - SigLIP attention, 16 heads x 72 per view, 256 keys (pi0_infer.py:588-596).
 //
 // Both compute the transposed logits S^T = K Q^T so that each lane holds 16 keys of ONE query row:
@@ -31,13 +34,29 @@ RTVLA_DEVICE bf16x8 cat44(bf16x4 lo, bf16x4 hi) {
     return v;
 }
 
-template <int WAVES, int MQ, int NTK>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(1, 1)))
+// where element (row, d) of the output goes: row-major [token][ld_tok] with the G heads of a token side by side (and the
+// batch index split into an outer and an inner part with a stride each), or the fragment-tiled [tokens][32 out_cols32]
+// matrix the action-expert O projection reads
+RTVLA_DEVICE bf16_t* attn_out_ptr(const AttnP& p, int batch, int row, int d, int hd) {
+    const int tok = row / p.group, sub = row - tok * p.group;
+    if (p.out_tiled) return p.out + ft_index(tok, batch * p.out_bcol + sub * hd + d, p.out_cols32);
+    const int bo = batch / p.batch_inner, bi = batch - bo * p.batch_inner;
+    return p.out + (size_t)bo * p.out_ostride + (size_t)bi * p.out_istride + (size_t)tok * p.ld_tok + sub * hd + d;
+}
+
+template <int WAVES, int MQ, int NTK, int HD>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(1, HD == 256 ? 1 : 2)))
 void mqa_kernel(AttnP p) {
+    constexpr int KD = HD / 32;                                       // 32-wide steps of the Q K^T contraction
+    constexpr int DT = HD / 16;                                       // 16-wide tiles of the output
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    f32x4* obuf = (f32x4*)smem_raw;                                   // [WAVES][16][64]
-    float* ms = (float*)(smem_raw + (size_t)WAVES * 16 * 64 * 16);    // [WAVES][MQ][16]
+    f32x4* obuf = (f32x4*)smem_raw;                                   // [WAVES][DT][64]
+    float* ms = (float*)(smem_raw + (size_t)WAVES * DT * 64 * 16);    // [WAVES][MQ][16]
     float* ls = ms + WAVES * MQ * 16;                                 // [WAVES][MQ][16]
+    const int batch = blockIdx.y;
+    const bf16_t* const qbase = p.q + (size_t)batch * p.q_bstride;
+    const bf16_t* const kbase = p.k + (size_t)batch * p.k_bstride;
+    const bf16_t* const vbase = p.vt + (size_t)batch * p.vt_bstride;
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
@@ -57,41 +76,43 @@ void mqa_kernel(AttnP p) {
     int vl = p.prefix_alloc;
     if (p.valid_len) vl = max(0, min(*p.valid_len, p.prefix_alloc));
 
-    bf16x8 qf[MQ][8];
+    bf16x8 qf[MQ][KD];
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         // fragment-tiled Q: one contiguous 1 KB read per fragment (row tiles past the end are padding)
-        const bf16_t* qp = p.q + ((size_t)(rowblk * MQ + mq) * 8 * 64 + lane) * 8;
+        const bf16_t* qp = qbase + ((size_t)(rowblk * MQ + mq) * KD * 64 + lane) * 8;
 #pragma unroll
-        for (int kd = 0; kd < 8; ++kd) qf[mq][kd] = *(const bf16x8*)(qp + kd * 512);
+        for (int kd = 0; kd < KD; ++kd) qf[mq][kd] = *(const bf16x8*)(qp + kd * 512);
     }
-    f32x4 o[MQ][16];
+    f32x4 o[MQ][DT];
     float mrun[MQ], lrun[MQ];
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         mrun[mq] = NEG_BIG; lrun[mq] = 0.f;
 #pragma unroll
-        for (int dt = 0; dt < 16; ++dt) o[mq][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int dt = 0; dt < DT; ++dt) o[mq][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     constexpr int KBS = NTK * 16;                    // keys per block
-    const int nkb = (p.keys + KBS - 1) / KBS;
+    int nkb = (p.keys + KBS - 1) / KBS;
+    // causal: the last row of this block sees keys up to its own token
+    if (p.causal) nkb = min(nkb, (min(m0 + 16 * MQ, p.rows) - 1) / p.group / KBS + 1);
     const int kb_begin = split * p.kb_per_split, kb_end = min(nkb, kb_begin + p.kb_per_split);
     const int keys32 = p.ldvt >> 5;
-    bf16x8 kf[NTK][8];        // K fragments of one key block (A operand of S^T = K Q^T)
-    bf16x8 vf[16][NTK / 2];      // V^T fragments of the block, in the key order the P registers have
+    bf16x8 kf[NTK][KD];       // K fragments of one key block (A operand of S^T = K Q^T)
+    bf16x8 vf[DT][NTK / 2];      // V^T fragments of the block, in the key order the P registers have
     auto load_k = [&](int kb) {
 #pragma unroll
         for (int nt = 0; nt < NTK; ++nt) {
-            const bf16_t* kp = p.k + ((size_t)(kb * NTK + nt) * 8 * 64 + lane) * 8;
+            const bf16_t* kp = kbase + ((size_t)(kb * NTK + nt) * KD * 64 + lane) * 8;
 #pragma unroll
-            for (int kd = 0; kd < 8; ++kd) kf[nt][kd] = *(const bf16x8*)(kp + kd * 512);
+            for (int kd = 0; kd < KD; ++kd) kf[nt][kd] = *(const bf16x8*)(kp + kd * 512);
         }
     };
     auto load_v = [&](int kb) {
 #pragma unroll
-        for (int dt = 0; dt < 16; ++dt) {
-            const bf16_t* vp = p.vt + ((size_t)(dt * keys32 + kb * (NTK / 2)) * 64 + lane) * 8;
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16_t* vp = vbase + ((size_t)(dt * keys32 + kb * (NTK / 2)) * 64 + lane) * 8;
 #pragma unroll
             for (int kk = 0; kk < NTK / 2; ++kk) vf[dt][kk] = *(const bf16x8*)(vp + kk * 512);
         }
@@ -110,7 +131,7 @@ void mqa_kernel(AttnP p) {
 #pragma unroll
         for (int nt = 0; nt < NTK; ++nt)
 #pragma unroll
-            for (int kd = 0; kd < 8; ++kd)
+            for (int kd = 0; kd < KD; ++kd)
 #pragma unroll
                 for (int mq = 0; mq < MQ; ++mq) st[mq][nt] = mfma16(kf[nt][kd], qf[mq][kd], st[mq][nt]);
         __builtin_amdgcn_sched_barrier(0);
@@ -130,6 +151,7 @@ void mqa_kernel(AttnP p) {
                     bool ok = key < p.keys;
                     if (key < p.prefix_alloc) ok = ok && key < vl;
                     else ok = ok && (row >= p.state_rows || key == p.prefix_alloc);
+                    if (p.causal) ok = ok && key <= row / p.group;
                     vis[nt][v] = ok;
                     const float s = ok ? st[mq][nt][v] * p.scale : NEG_BIG;
                     st[mq][nt][v] = s;
@@ -153,12 +175,12 @@ void mqa_kernel(AttnP p) {
             lrun[mq] = lrun[mq] * alpha + sum;
             mrun[mq] = mnew;
 #pragma unroll
-            for (int dt = 0; dt < 16; ++dt) o[mq][dt] *= alpha;
+            for (int dt = 0; dt < DT; ++dt) o[mq][dt] *= alpha;
 #pragma unroll
             for (int kk = 0; kk < NTK / 2; ++kk) pb[mq][kk] = cat44(pack4(st[mq][2 * kk]), pack4(st[mq][2 * kk + 1]));
         }
 #pragma unroll
-        for (int dt = 0; dt < 16; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int kk = 0; kk < NTK / 2; ++kk) {
 #pragma unroll
@@ -184,36 +206,33 @@ void mqa_kernel(AttnP p) {
         const float sc = __expf(mrun[mq] - mg);
         lrun[mq] *= sc;
 #pragma unroll
-        for (int dt = 0; dt < 16; ++dt) o[mq][dt] *= sc;
+        for (int dt = 0; dt < DT; ++dt) o[mq][dt] *= sc;
         if (g == 0) ls[(w * MQ + mq) * 16 + r] = lrun[mq];
         mgl[mq] = mg;
     }
-    // partial record of one (row block, split): MQ x { O [16][64] f32x4 | max [16] | sum [16] }
-    constexpr int REC = 16 * 64 * 4 + 32;
+    // partial record of one (row block, split): MQ x { O [DT][64] f32x4 | max [16] | sum [16] }
+    constexpr int REC = DT * 64 * 4 + 32;
     float* const mine = p.partial + ((size_t)rowblk * nsplit + split) * (MQ * REC);
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         __syncthreads();                       // ls written / previous obuf round consumed
 #pragma unroll
-        for (int dt = 0; dt < 16; ++dt) obuf[((size_t)w * 16 + dt) * 64 + lane] = o[mq][dt];
+        for (int dt = 0; dt < DT; ++dt) obuf[((size_t)w * DT + dt) * 64 + lane] = o[mq][dt];
         __syncthreads();
         float lt = 0.f;
 #pragma unroll
         for (int ww = 0; ww < WAVES; ++ww) lt += ls[(ww * MQ + mq) * 16 + r];
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         const int row = m0 + mq * 16 + r;
-        if (nsplit > 1 && w == 0 && g == 0) { mine[mq * REC + 4096 + r] = mgl[mq]; mine[mq * REC + 4112 + r] = lt; }
-        for (int dt = w; dt < 16; dt += WAVES) {
+        if (nsplit > 1 && w == 0 && g == 0) { mine[mq * REC + DT * 256 + r] = mgl[mq]; mine[mq * REC + DT * 256 + 16 + r] = lt; }
+        for (int dt = w; dt < DT; dt += WAVES) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ww = 0; ww < WAVES; ++ww) t += obuf[((size_t)ww * 16 + dt) * 64 + lane];
+            for (int ww = 0; ww < WAVES; ++ww) t += obuf[((size_t)ww * DT + dt) * 64 + lane];
             if (nsplit > 1) {
                 *(f32x4*)(mine + mq * REC + (dt * 64 + lane) * 4) = t;
             } else if (row < p.rows) {
-                const int d = dt * 16 + 4 * g;
-                // tiled output: the [tokens][8*256] matrix the suffix O-projection reads as MFMA fragments
-                bf16_t* dst = p.out_tiled ? p.out + ft_index(row >> 3, (row & 7) * 256 + d, 64) : p.out + (size_t)row * p.ldo + d;
-                store4(dst, pack4(t * inv));
+                store4(attn_out_ptr(p, batch, row, dt * 16 + 4 * g, HD), pack4(t * inv));
             }
         }
     }
@@ -254,8 +273,7 @@ void attn_merge_kernel(AttnP p, int nsplit) {
         const int row = (rb * MQ + mq) * 16 + r;
         if (row < p.rows) {
             const int d = dt * 16 + 4 * g;
-            bf16_t* dst = p.out_tiled ? p.out + ft_index(row >> 3, (row & 7) * 256 + d, 64) : p.out + (size_t)row * p.ldo + d;
-            store4(dst, pack4(t * inv));
+            store4(attn_out_ptr(p, 0, row, d, 256), pack4(t * inv));
         }
     }
 }
@@ -342,10 +360,10 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     }
 }
 
-template <int WAVES, int MQ, int NTK>
+template <int WAVES, int MQ, int NTK, int HD>
 int launch_mqa_inst(AttnP p, hipStream_t s) {
-    const size_t smem = (size_t)WAVES * 16 * 64 * 16 + (size_t)2 * WAVES * MQ * 16 * 4;
-    auto kern = mqa_kernel<WAVES, MQ, NTK>;
+    const size_t smem = (size_t)WAVES * (HD / 16) * 64 * 16 + (size_t)2 * WAVES * MQ * 16 * 4;
+    auto kern = mqa_kernel<WAVES, MQ, NTK, HD>;
     if (smem > 65536) {
         static bool done = false;
         if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
@@ -356,11 +374,11 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
     p.kb_per_split = (nkb + want - 1) / want;
     const int nsplit = (nkb + p.kb_per_split - 1) / p.kb_per_split;
     if (nsplit > 1) {
-        if (!p.partial || nsplit > 16) return 1;
+        if (!p.partial || nsplit > 16 || HD != 256 || p.batch > 1) return 1;      // the key split over workgroups exists for the Gemma suffix pass only
         if ((size_t)blocks * nsplit * MQ * (16 * 64 * 4 + 32) > p.partial_floats) return 3;
     }
     p.nsplit_eff = nsplit;
-    hipLaunchKernelGGL(kern, dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks), dim3(WAVES * 64), smem, s, p);
+    hipLaunchKernelGGL(kern, dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(WAVES * 64), smem, s, p);
     if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
     else if (nsplit > 1) hipLaunchKernelGGL((attn_merge_kernel<MQ, 8>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
     return hipGetLastError() == hipSuccess ? 0 : 5;
@@ -368,11 +386,18 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
 
 }  // namespace
 
-int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s) {
-    if (p.rows <= 0 || p.keys <= 0 || (p.ldvt & 63) || p.ldvt < ((p.keys + 63) / 64) * 64) return 1;
-    switch (variant) {                                          // template: waves, row tiles per workgroup, 16-key tiles per wave round
-        case ATTN_PREFIX: return launch_mqa_inst<4, 2, 2>(p, s);
-        case ATTN_SUFFIX: return launch_mqa_inst<4, 1, 2>(p, s);
+int launch_mqa_attention(const AttnP& p0, int variant, hipStream_t s) {
+    AttnP p = p0;
+    if (p.rows <= 0 || p.keys <= 0 || (p.ldvt & 31) || p.ldvt < ((p.keys + 31) / 32) * 32) return 1;
+    if (p.batch < 1) p.batch = 1;
+    if (p.batch_inner < 1) p.batch_inner = 1;
+    if (p.group < 1) return 1;
+    switch (variant) {                                          // template: waves, row tiles per workgroup, 16-key tiles per wave round, head width
+        case ATTN_PREFIX: return launch_mqa_inst<4, 2, 2, 256>(p, s);
+        case ATTN_SUFFIX: return launch_mqa_inst<4, 1, 2, 256>(p, s);
+        case ATTN_GQA128_PREFIX: return launch_mqa_inst<4, 2, 2, 128>(p, s);
+        case ATTN_GQA128_SUFFIX: return launch_mqa_inst<4, 1, 2, 128>(p, s);
+        case ATTN_VIT64: return launch_mqa_inst<4, 4, 2, 64>(p, s);
     }
     return 2;
 }

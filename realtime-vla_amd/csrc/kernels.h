@@ -111,13 +111,20 @@ void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t
 
 // ----- attention --------------------------------------------------------------------------
 struct AttnP {
-    const bf16_t* q;                 // fragment-tiled [rows padded to the workgroup tile][256]
-    const bf16_t* k;                 // fragment-tiled [keys padded to 64][256]
-    const bf16_t* vt; int ldvt;      // permuted-key tiled V^T [256][ldvt], ldvt = keys padded to 64
-    bf16_t* out; int ldo;            // row-major or fragment-tiled [rows][256] (out_tiled)
-    int out_tiled;
+    // query rows are token * group + head for the `group` query heads that share the K/V head; HD = head width
+    const bf16_t* q;                 // fragment-tiled [rows padded to the workgroup tile][HD]
+    const bf16_t* k;                 // fragment-tiled [keys padded to 32][HD]
+    const bf16_t* vt; int ldvt;      // permuted-key tiled V^T [HD][ldvt], ldvt = keys padded to 32
+    int batch; size_t q_bstride, k_bstride, vt_bstride;        // independent K/V heads (blockIdx.y) and their strides, in elements
+    int group;
+    // output element (row, d): row-major  out[bo * out_ostride + bi * out_istride + token * ld_tok + head * HD + d]  with the batch
+    // index split as bo * batch_inner + bi, or (out_tiled) the fragment-tiled [tokens][32 out_cols32] matrix at column
+    // batch * out_bcol + head * HD + d
+    bf16_t* out; int ld_tok; int batch_inner; size_t out_ostride, out_istride;
+    int out_tiled, out_bcol, out_cols32;
     int rows, keys;
     float scale;
+    int causal;                      // key j visible to row r only if j <= r / group (keys and tokens count from the same origin)
     // masking: key j is visible to row r iff
     //   j < prefix_alloc ? j < *valid_len (or prefix_alloc if valid_len == null)
     //                    : (r >= state_rows || j == prefix_alloc)
@@ -127,7 +134,9 @@ struct AttnP {
     int kb_per_split, nsplit_eff;    // filled by the launcher
     RTVLA_KO_FIELD
 };
-enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1 };    // many rows, two row tiles per workgroup / few rows, one row tile and a key split
+// Gemma (HD 256): many rows, two row tiles per workgroup / few rows, one row tile and a key split; DM0 grouped-query (HD 128)
+// prefix and suffix; DM0 ViT (HD 64)
+enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1, ATTN_GQA128_PREFIX, ATTN_GQA128_SUFFIX, ATTN_VIT64 };
 int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s);
 // SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major
 void launch_vision_attention(const bf16_t* q, const bf16_t* k, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);

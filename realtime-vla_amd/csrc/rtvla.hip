@@ -408,7 +408,7 @@ struct Sched {
         if (i == L - 1) return;                      // the last layer only fills the KV cache
         AttnP a{};
         a.q = c->B("encoder_Q"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
-        a.out = c->B("encoder_attn"); a.ldo = 256; a.out_tiled = 0; a.rows = 8 * S_e; a.keys = S_e; a.scale = 0.0625f;
+        a.out = c->B("encoder_attn"); a.group = 8; a.ld_tok = 2048; a.out_tiled = 0; a.rows = 8 * S_e; a.keys = S_e; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = 0;
         if (c->want("prefix attn")) c->note(launch_mqa_attention(a, ATTN_PREFIX, s), "prefix attn");
         gemm(c->B("encoder_attn"), 2048, S_e, S_e, c->TW("t_encoder_attn_o_w", i), nullptr, 2048, 2048, EPI_PARTIAL, GemmP{}, "prefix o");
@@ -467,7 +467,7 @@ struct Sched {
         skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_attn_qkv_w", i), nullptr, 1024, 2560, norm, st_attn, SK_QKV_ROPE, q, "suffix qkv");
         AttnP a{};
         a.q = c->B("decoder_q_buf"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
-        a.out = c->B("decoder_attn"); a.ldo = 256; a.out_tiled = 1; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
+        a.out = c->B("decoder_attn"); a.group = 8; a.out_tiled = 1; a.out_cols32 = 64; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
         a.nsplit = c->attn_split > 0 ? c->attn_split : std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
         if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_SUFFIX, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
