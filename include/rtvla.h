@@ -35,7 +35,7 @@ enum rtvla_status {
     RTVLA_ERR_LIMIT = 7       /* shape outside the supported range                         */
 };
 
-enum rtvla_model { RTVLA_PI0 = 0, RTVLA_PI05 = 1 };
+enum rtvla_model { RTVLA_PI0 = 0, RTVLA_PI05 = 1, RTVLA_DM0 = 2 };
 
 /* Static shape set of one inference object.
  * Replaces the constructor arguments and literals of Pi0Inference.__init__

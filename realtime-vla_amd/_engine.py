@@ -9,6 +9,7 @@ import rtvla_capi as capi
 from tile_cache import TileCache, fingerprint
 
 _DTYPES = {2: torch.bfloat16, 4: torch.int32}
+_ANY_ROWS = ("vision_embed_tokens_w",)          # tables whose row count is whatever the checkpoint holds
 
 
 def rope_table(start, count, device):
@@ -23,30 +24,34 @@ def rope_table(start, count, device):
 
 
 class Engine:
-    def __init__(self, model, checkpoint, num_views, prompt_len, chunk_size, num_steps=10, skip_keys=(), tile_cache=None):
+    def __init__(self, model, checkpoint, num_views, prompt_len, chunk_size, num_steps=10, skip_keys=(), tile_cache=None,
+                 vision_layers=None, llm_layers=None):
         if not torch.cuda.is_available():
             raise RuntimeError("realtime-vla_amd needs a ROCm GPU (MI355X / gfx950); there is no CPU path")
         self.device = torch.device("cuda", torch.cuda.current_device())
-        vision_layers, llm_layers = 27, 18
-        if "vision_attn_qkv_w" in checkpoint:
-            vision_layers = int(checkpoint["vision_attn_qkv_w"].shape[0])
-        if "encoder_attn_qkv_w" in checkpoint:
-            llm_layers = int(checkpoint["encoder_attn_qkv_w"].shape[0])
+        if vision_layers is None:
+            vision_layers = int(checkpoint["vision_attn_qkv_w"].shape[0]) if "vision_attn_qkv_w" in checkpoint else 27
+        if llm_layers is None:
+            llm_layers = int(checkpoint["encoder_attn_qkv_w"].shape[0]) if "encoder_attn_qkv_w" in checkpoint else 18
         self.model, self.vision_layers, self.llm_layers = model, vision_layers, llm_layers
         self.tile_cache = TileCache(tile_cache) if isinstance(tile_cache, (str, os.PathLike)) else tile_cache
         self.tile_cache_hit = None                                   # True / False after prepare() when a cache is in use
         self.ctx = capi.Context(model, num_views, prompt_len, chunk_size, num_steps, vision_layers, llm_layers)
         self.weights, self.buffers = {}, {}
         for name, elem, shape, is_weight, required in self.ctx.tensors():
-            if is_weight and not required:
-                # optional weights (Pi05 embedding table, ~1 GB) exist only when the checkpoint brings them
+            dtype = torch.float32 if (is_weight and elem == 4) else _DTYPES[elem]      # 4-byte weights are fp32, 4-byte io buffers int32
+            if is_weight and (not required or name in _ANY_ROWS):
+                # optional weights (Pi05 embedding table, ~1 GB) exist only when the checkpoint brings them; the token
+                # embedding tables take their row count from the checkpoint
                 if name in checkpoint and name not in skip_keys:
                     v = torch.as_tensor(checkpoint[name])
-                    self.weights[name] = torch.zeros(*v.shape, dtype=_DTYPES[elem], device=self.device)
+                    self.weights[name] = torch.zeros(*v.shape, dtype=dtype, device=self.device)
+                elif required:
+                    self.weights[name] = torch.zeros(1, shape[1], dtype=dtype, device=self.device)
                 continue
             # zero-initialised so that a weight the checkpoint omits (the reference leaves it
             # uninitialised, benchmark.py:9-11) can never inject NaN/Inf
-            t = torch.zeros(*shape, dtype=_DTYPES[elem], device=self.device)
+            t = torch.zeros(*shape, dtype=dtype, device=self.device)
             (self.weights if is_weight else self.buffers)[name] = t
         for k, v in checkpoint.items():
             if k in skip_keys:

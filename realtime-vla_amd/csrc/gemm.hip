@@ -15,7 +15,7 @@
 
 namespace {
 
-template <int EPI> struct EpiTraits { static constexpr bool dual = (EPI == EPI_GEGLU); };
+template <int EPI> struct EpiTraits { static constexpr bool dual = (EPI == EPI_GEGLU || EPI == EPI_SWIGLU); };
 
 RTVLA_DEVICE f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 
@@ -202,7 +202,7 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
     // ---- epilogue: lane (h, r) holds rows m = m0 + 32 i + r, columns n = 32 tile + 8 grp + 4 h + e ----
     // Row-major outputs go through LDS one 32-row tile at a time so that the global stores are whole
     // 16-byte chunks of contiguous row segments (256 B - 1 KB per row) instead of 8-byte pieces of 32 rows.
-    constexpr bool ROWMAJOR = (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_PATCH || EPI == EPI_GEGLU || EPI == EPI_PARTIAL);
+    constexpr bool ROWMAJOR = (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_PATCH || EPI == EPI_GEGLU || EPI == EPI_SWIGLU || EPI == EPI_PARTIAL);
     if constexpr (ROWMAJOR) {
         constexpr int ESZ = (EPI == EPI_PARTIAL) ? 4 : 2;
         constexpr int OUTW = WN * HALF * 32;                       // output columns of the workgroup
@@ -239,10 +239,18 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
                         if (KO(p, 4)) *(bf16x4*)dst = pack4(v[0] * u[0], v[1] * u[1], v[2] * u[2], v[3] * u[3]);      // (KO 4: no GELU)
                         else
                         *(bf16x4*)dst = pack4(gelu_tanh(v[0]) * u[0], gelu_tanh(v[1]) * u[1], gelu_tanh(v[2]) * u[2], gelu_tanh(v[3]) * u[3]);
+                    } else if constexpr (EPI == EPI_SWIGLU) {
+                        const float f = p.rowscale[min(m, p.M - 1)];
+                        f32x4 u = {acc[i][j + HALF][4 * grp], acc[i][j + HALF][4 * grp + 1], acc[i][j + HALF][4 * grp + 2], acc[i][j + HALF][4 * grp + 3]};
+                        v *= f; u *= f;
+                        *(bf16x4*)dst = pack4(siluf(v[0]) * u[0], siluf(v[1]) * u[1], siluf(v[2]) * u[2], siluf(v[3]) * u[3]);
                     } else {
-                        const bf16x4 b = load4(p.bias + n0);
+                        if (p.bias_f32) v += *(const f32x4*)(p.bias_f32 + n0);
+                        else {
+                            const bf16x4 b = load4(p.bias + n0);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] += bf2f(b[e]);
+                            for (int e = 0; e < 4; ++e) v[e] += bf2f(b[e]);
+                        }
                         if constexpr (EPI == EPI_PATCH) {
                             const bf16x4 rs = load4(p.res + (size_t)(min(m, p.M - 1) % p.res_mod) * p.ldr + n0);
 #pragma unroll
@@ -325,6 +333,26 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
                     const int d = n0 - 2304;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) p.vt[vt_index(d + e, m, p.ldvt >> 5)] = f2bf(v[e]);
+                }
+            } else if constexpr (EPI == EPI_VIT_QKV_ROPE) {
+                // DM0 ViT (dm0_infer.py:589-598): + fp32 bias, rounded to bf16 as the reference's QKV buffer is, then the 2-D rotary
+                // embedding on Q and K; per (image, head) Q and K as fragment-tiled [seq_pad][64], V^T as [64][seq_pad]
+                v += *(const f32x4*)(p.bias_f32 + n0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = round_bf16(v[e]);
+                const int which = n0 >> 10, cc = n0 & 1023, head = cc >> 6, d = cc & 63;
+                const int img = m / p.seq, tok = m - img * p.seq;
+                const size_t vh = (size_t)(img * 16 + head);
+                if (which < 2) {
+                    const bf16x4 cs = load4(p.rope + (size_t)tok * 64 + d);
+                    const float c0 = bf2f(cs[0]), s0 = bf2f(cs[1]), c1 = bf2f(cs[2]), s1 = bf2f(cs[3]);
+                    const f32x4 w = v;
+                    v[0] = w[0] * c0 - w[1] * s0; v[1] = w[1] * c0 + w[0] * s0;
+                    v[2] = w[2] * c1 - w[3] * s1; v[3] = w[3] * c1 + w[2] * s1;
+                    store4((which == 0 ? p.q : p.k) + vh * ((size_t)p.seq_pad * 64) + ft_index(tok, d, 2), pack4(v));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) p.vt[vh * ((size_t)64 * p.seq_pad) + vt_index(d + e, tok, p.seq_pad >> 5)] = f2bf(v[e]);
                 }
             } else if constexpr (EPI == EPI_VIS_QKV) {
                 const bf16x4 b = load4(p.bias + n0);
@@ -429,6 +457,8 @@ int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {
         case EPI_PARTIAL:   return launch_epi<EPI_PARTIAL>(p, tile, s);
         case EPI_QKV_ROPE:  return launch_epi<EPI_QKV_ROPE>(p, tile, s);
         case EPI_VIS_QKV:   return launch_epi<EPI_VIS_QKV>(p, tile, s);
+        case EPI_SWIGLU:    return launch_epi<EPI_SWIGLU>(p, tile, s);
+        case EPI_VIT_QKV_ROPE: return launch_epi<EPI_VIT_QKV_ROPE>(p, tile, s);
     }
     return 2;
 }

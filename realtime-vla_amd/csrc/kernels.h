@@ -34,6 +34,7 @@ static inline size_t tiled_elems(int K, int N, int G = 1) { return (size_t)((n16
 static inline size_t tiled_elems_wide(int K, int N, int G) { return (size_t)(((N + 31) / 32 + G - 1) / G) * G * k32_padded(K) * 2 * 512; }
 
 void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide, hipStream_t s);
+void launch_pretile_padded(const bf16_t* W, int K, int K_pad, int N, bf16_t* out, hipStream_t s);
 
 // ----- large-M MFMA GEMM --------------------------------------------------------------
 enum GemmEpilogue {
@@ -44,6 +45,8 @@ enum GemmEpilogue {
     EPI_PARTIAL,       // fp32 split-K partial
     EPI_QKV_ROPE,      // Gemma prefix: bf16 -> interleaved RoPE on Q,K -> Q / K cache / transposed V cache
     EPI_VIS_QKV,       // SigLIP: +bias, Q|K row-major, V transposed per (view, head)
+    EPI_SWIGLU,        // out = silu(acc(B0) * rowscale[row]) * (acc(B1) * rowscale[row])   (DM0 prefix MLP)
+    EPI_VIT_QKV_ROPE,  // DM0 ViT: +bias, bf16, 2-D rotary on Q and K (16 heads x 64), Q / K / V^T per (image, head)
 };
 
 struct GemmP {
@@ -54,6 +57,9 @@ struct GemmP {
     int nsplit;                                // split-K factor (EPI_PARTIAL only when > 1)
     bf16_t* out; int ldo;
     const bf16_t* bias;
+    const float* bias_f32;                     // fp32 bias instead of `bias` (DM0's folded LayerNorm biases)
+    const float* rowscale;                     // per-row factor applied to the accumulators (EPI_SWIGLU)
+    int seq, seq_pad;                          // EPI_VIT_QKV_ROPE: tokens per image and their padded count in the Q / K / V^T tiles
     const bf16_t* res; int ldr; int res_mod;
     float* partial; int ldp; size_t pstride;   // [split][row][ldp]
     const bf16_t* rope;                        // [row][256] = cos0 sin0 cos1 sin1 ...
@@ -77,6 +83,7 @@ struct ReduceP {
     bf16_t* xn; int ldxn;                       // normalised copy (may be null)
     int M, N;
     int norm; const bf16_t* nw; const bf16_t* nb; float eps;
+    float* factor;                              // NORM_RMS: the row's rsqrt(mean x^2 + eps) as fp32 (may be null; xn may then be null too)
 };
 int launch_reduce(const ReduceP& p, hipStream_t s);
 
@@ -87,6 +94,7 @@ enum SkinnyEpilogue {
     SK_RES,            // out += acc (* gate[col])
     SK_QKV_ROPE,       // RoPE + scatter to Q / K cache rows / transposed V cache columns
     SK_GEGLU,          // out = gelu_tanh(acc(B0)) * acc(B1)
+    SK_SWIGLU,         // out = silu(acc(B0)) * acc(B1)
 };
 enum SkinnyNorm { SN_NONE = 0, SN_RMS, SN_ADARMS };
 struct SkinnyP {
@@ -96,6 +104,7 @@ struct SkinnyP {
     const bf16_t* B0; const bf16_t* B1; int K; int N16; int K32p;
     int norm; const bf16_t* style;             // SN_ADARMS: [scale | shift | gate] each K wide
     float eps;
+    int factor_f32;                            // SN_RMS: keep the row factor in fp32 (DM0) instead of rounding it to bf16 (Pi0)
     bf16_t* out; int ldo;
     const bf16_t* bias; const bf16_t* gate;    // per-column
     const bf16_t* rope;                        // [row][256]
@@ -147,5 +156,15 @@ void launch_prompt_stage(const bf16_t* emb, int vocab, const int* ids, const int
 void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hipStream_t s);
 void launch_copy_rows(const bf16_t* src, int lds, bf16_t* dst, int ldd, int rows, int cols, hipStream_t s);
 void launch_fill_zero(void* p, size_t bytes, hipStream_t s);
+void launch_fill_bf16(bf16_t* p, size_t n, float v, hipStream_t s);
+
+// ----- DM0 (csrc/dm0.hip) ---------------------------------------------------------------------
+void launch_dm0_im2col_nchw(const bf16_t* images, bf16_t* patches, int ldp, int n_images, hipStream_t s);
+void launch_dm0_embed_ln(const bf16_t* conv, const bf16_t* cls, const bf16_t* pos, const bf16_t* w, const bf16_t* b, bf16_t* x, int n_images, hipStream_t s);
+void launch_dm0_im2col3x3(const bf16_t* in, int img_rows, int row0, int in_h, int in_w, int C, bf16_t* col, int n_images, hipStream_t s);
+void launch_dm0_gather_rows(const bf16_t* table, int table_rows, const int* ids, bf16_t* dst, int rows, hipStream_t s);
+void launch_dm0_qknorm_rope(const bf16_t* qkv, int ld, const float* factor, const bf16_t* x_tiled, const bf16_t* qw, const bf16_t* kw, const bf16_t* rope,
+                            bf16_t* q, size_t q_bstride, bf16_t* k, size_t k_bstride, bf16_t* vt, size_t vt_bstride, int keys32, int key_row0, int rows,
+                            hipStream_t s);
 void launch_scale_inplace(bf16_t* p, size_t n, float f, hipStream_t s);
 void launch_copy_bytes(const void* src, void* dst, size_t bytes, hipStream_t s);

@@ -73,10 +73,13 @@ void reduce_kernel(ReduceP p) {
     const float inv_n = 1.0f / (float)p.N;
     if (NORM == NORM_RMS) {
         const float f = rsqrtf(tot * inv_n + p.eps);
+        if (p.factor && tid == 0) p.factor[m] = f;
+        if (p.xn) {
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            const int c = tid + it * 256;
-            if (c < nq) store4(p.xn + (size_t)m * p.ldxn + c * 4, pack4(v[it] * f));
+            for (int it = 0; it < 2; ++it) {
+                const int c = tid + it * 256;
+                if (c < nq) store4(p.xn + (size_t)m * p.ldxn + c * 4, pack4(v[it] * f));
+            }
         }
     } else {
         const float mean = tot * inv_n;
@@ -200,6 +203,13 @@ void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide,
     hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, KBp, G, wide, chunks);
 }
 
+// W has K rows; the tiles are laid out as for K_pad rows (a multiple of 128), the rows past K zero: for a kernel that only takes
+// the padded K
+void launch_pretile_padded(const bf16_t* W, int K, int K_pad, int N, bf16_t* out, hipStream_t s) {
+    const size_t chunks = tiled_elems(K_pad, N, 1) / 8;
+    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, k32_padded(K_pad), 1, 0, chunks);
+}
+
 template <int NORM>
 static int launch_reduce_norm(const ReduceP& p, hipStream_t s) {
     const dim3 grid(p.M), block(256);
@@ -218,7 +228,8 @@ static int launch_reduce_norm(const ReduceP& p, hipStream_t s) {
 
 int launch_reduce(const ReduceP& p, hipStream_t s) {
     if (p.M <= 0 || p.N <= 0 || (p.N & 3) || p.N > 2048) return 1;
-    if (p.norm != NORM_NONE && !p.xn) return 1;
+    if (p.norm == NORM_LAYER && !p.xn) return 1;
+    if (p.norm == NORM_RMS && !p.xn && !p.factor) return 1;
     if (p.norm == NORM_LAYER && (!p.nw || !p.nb)) return 1;
     switch (p.norm) {
         case NORM_NONE:  return launch_reduce_norm<NORM_NONE>(p, s);

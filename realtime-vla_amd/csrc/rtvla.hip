@@ -312,6 +312,119 @@ int build_tables(rtvla_ctx* c) {
     return 0;
 }
 
+// DM0 (/root/reference/dm0_infer.py:965-1076): tensors under the reference's names, then the workspace.
+constexpr int DM0_SEQ = 2705;          // 52 x 52 patches + class token per image
+constexpr int DM0_SEQ_PAD = 2720;      // padded to the 32-key blocks of the attention kernel
+constexpr int DM0_TOK = 169;           // tokens per image after the two stride-2 convolutions
+
+int build_tables_dm0(rtvla_ctx* c) {
+    const rtvla_dims& d = c->d;
+    const int64_t V = d.vision_layers, L = d.llm_layers, n = d.num_views, P = c->S_e, ch = d.chunk_size;
+    c->add_tensor("decoder_attn_qkv_w", true, 2, {L, 1024, 4096});
+    c->add_tensor("decoder_q_norm_w", true, 2, {L, 128});
+    c->add_tensor("decoder_k_norm_w", true, 2, {L, 128});
+    c->add_tensor("decoder_attn_o_w", true, 2, {L, 2048, 1024});
+    c->add_tensor("decoder_ffn_gate_w", true, 2, {L, 1024, 1536});
+    c->add_tensor("decoder_ffn_up_w", true, 2, {L, 1024, 1536});
+    c->add_tensor("decoder_ffn_down_w", true, 2, {L, 1536, 1024});
+    c->add_tensor("decoder_action_fused_in_proj_w", true, 2, {32, 1024});
+    c->add_tensor("decoder_action_fused_time_biases", true, 2, {10, 1024});
+    c->add_tensor("decoder_action_mlp_w", true, 2, {1024, 1024});
+    c->add_tensor("decoder_action_mlp_b", true, 2, {1024});
+    c->add_tensor("decoder_action_fused_out_proj_w", true, 2, {1024, 32});
+    c->add_tensor("decoder_action_fused_out_proj_b", true, 2, {32});
+    c->add_tensor("llm_attn_qkv_w", true, 2, {L, 2048, 4096});
+    c->add_tensor("llm_q_norm_w", true, 2, {L, 128});
+    c->add_tensor("llm_k_norm_w", true, 2, {L, 128});
+    c->add_tensor("llm_attn_o_w", true, 2, {L, 2048, 2048});
+    c->add_tensor("llm_ffn_gate_w", true, 2, {L, 2048, 6144});
+    c->add_tensor("llm_ffn_up_w", true, 2, {L, 2048, 6144});
+    c->add_tensor("llm_ffn_down_w", true, 2, {L, 6144, 2048});
+    c->add_tensor("vision_conv1_w_t", true, 2, {588, 1024});
+    c->add_tensor("vision_class_embedding", true, 2, {1024});
+    c->add_tensor("vision_pos_emb", true, 2, {DM0_SEQ, 1024});
+    c->add_tensor("vision_ln_pre_w", true, 2, {1024});
+    c->add_tensor("vision_ln_pre_b", true, 2, {1024});
+    c->add_tensor("vision_fused_qkv_w", true, 2, {V, 1024, 3072});
+    c->add_tensor("vision_fused_qkv_b", true, 4, {V, 3072});          // fp32 (weights of 4-byte elements are fp32)
+    c->add_tensor("vision_qkv_col_sum", true, 4, {V, 3072});          // bound for the reference's key set; the LayerNorm is applied to the rows instead
+    c->add_tensor("vision_out_proj_w", true, 2, {V, 1024, 1024});
+    c->add_tensor("vision_out_proj_b", true, 2, {V, 1024});
+    c->add_tensor("vision_fused_fc_w", true, 2, {V, 1024, 4096});
+    c->add_tensor("vision_fused_fc_b", true, 4, {V, 4096});
+    c->add_tensor("vision_fc_col_sum", true, 4, {V, 4096});
+    c->add_tensor("vision_proj_w", true, 2, {V, 4096, 1024});
+    c->add_tensor("vision_proj_b", true, 2, {V, 1024});
+    c->add_tensor("vision_ds1_w", true, 2, {3, 3, 1024, 2048});
+    c->add_tensor("vision_ds1_b", true, 2, {2048});
+    c->add_tensor("vision_ds2_w", true, 2, {3, 3, 2048, 4096});
+    c->add_tensor("vision_ds2_b", true, 2, {4096});
+    c->add_tensor("vision_projector_w_t", true, 2, {4096, 2048});
+    c->add_tensor("vision_embed_tokens_w", true, 2, {152701, 2048});   // any row count, taken from the bound size
+    c->add_tensor("images", false, 2, {n, 3, 728, 728});
+    c->add_tensor("input_ids", false, 4, {d.prompt_len});              // int32
+    c->add_tensor("diffusion_noise", false, 2, {ch, 32});
+    c->add_tensor("prefix_rope_weights", false, 2, {P, 128});
+    c->add_tensor("decoder_rope_weights", false, 2, {ch, 128});
+    c->add_tensor("vision_rope", false, 2, {DM0_SEQ, 64});             // (cos, sin) per rotation pair of the 2-D rotary embedding
+
+    // ---- workspace: re-tiled weights first, then activations ----
+    c->add_tiled("t_vision_conv1_w_t", 588, 1024, 1, 8, 1);
+    c->add_tiled("t_vision_fused_qkv_w", 1024, 3072, V, 8, 1);
+    c->add_tiled("t_vision_out_proj_w", 1024, 1024, V, 8, 1);
+    c->add_tiled("t_vision_fused_fc_w", 1024, 4096, V, 8, 1);
+    c->add_tiled("t_vision_proj_w", 4096, 1024, V, 8, 1);
+    c->add_tiled("t_vision_ds1_w", 9216, 2048, 1, 8, 1);
+    c->add_tiled("t_vision_ds2_w", 18432, 4096, 1, 8, 1);
+    c->add_tiled("t_vision_projector_w_t", 4096, 2048, 1, 8, 1);
+    c->add_tiled("t_llm_attn_qkv_w", 2048, 4096, L, 8, 1);
+    c->add_tiled("t_llm_attn_o_w", 2048, 2048, L, 8, 1);
+    c->add_tiled("t_llm_ffn_gate_w", 2048, 6144, L, 4, 1);
+    c->add_tiled("t_llm_ffn_up_w", 2048, 6144, L, 4, 1);
+    c->add_tiled("t_llm_ffn_down_w", 6144, 2048, L, 8, 1);
+    c->add_tiled("t_decoder_attn_qkv_w", 1024, 4096, L);
+    c->add_tiled("t_decoder_attn_o_w", 2048, 1024, L);
+    c->add_tiled("t_decoder_ffn_gate_w", 1024, 1536, L);
+    c->add_tiled("t_decoder_ffn_up_w", 1024, 1536, L);
+    c->add_tiled("t_decoder_ffn_down_w", 2048, 1024, L);              // K = 1536 zero-padded to the 2048 the streaming kernel takes
+    c->add_tiled("t_decoder_action_mlp_w", 1024, 1024, 1);
+    c->add_tiled("t_decoder_out_proj_w", 1024, 32, 1);
+    c->act_begin = c->ws_bytes;
+    const int64_t M = n * DM0_SEQ;
+    c->add_buf("const_ones", 1, 1024, 1024);
+    c->add_buf("const_zeros", 1, 6144, 6144);
+    c->add_buf("vision_patches", n * 2704, PATCH_LD, PATCH_LD);
+    c->add_buf("vision_conv1_buf", n * 2704, 1024, 1024);
+    c->add_buf("vision_x_2d", M, 1024, 1024);
+    c->add_buf("vision_x_norm", M, 1024, 1024);
+    c->add_buf("vision_Q", n * 16, DM0_SEQ_PAD * 64, DM0_SEQ_PAD * 64);    // fragment-tiled [2720][64] per (image, head)
+    c->add_buf("vision_K", n * 16, DM0_SEQ_PAD * 64, DM0_SEQ_PAD * 64);
+    c->add_buf("vision_Vt", n * 16, 64 * DM0_SEQ_PAD, 64 * DM0_SEQ_PAD);   // tiled V^T [64][2720]
+    c->add_buf("vision_attn", M, 1024, 1024);
+    c->add_buf("vision_fc", M, 4096, 4096);
+    c->add_buf("vision_col1", n * 676, 9216, 9216);
+    c->add_buf("vision_mm1", n * 676, 2048, 2048);
+    c->add_buf("vision_col2", n * DM0_TOK, 18432, 18432);
+    c->add_buf("vision_mm2", n * DM0_TOK, 4096, 4096);
+    c->add_buf("prefix_x", P, 2048, 2048);
+    c->add_buf("prefix_qkv", P, 4096, 4096);
+    c->add_buf("prefix_Q", 8, ((2 * P + 31) / 32) * 32 * 128, ((2 * P + 31) / 32) * 32 * 128);     // per K/V head: fragment-tiled [token*2 + head][128]
+    c->add_buf("prefix_attn", P, 2048, 2048);
+    c->add_buf("prefix_hidden", P, 6144, 6144);
+    c->add_buf("prefix_norm_factor", 1, P, P, 4);
+    c->add_buf("kv_K", L * 8, c->keys_pad * 128, c->keys_pad * 128);       // per (layer, K/V head): fragment-tiled [keys_pad][128]
+    c->add_buf("kv_Vt", L * 8, 128 * c->keys_pad, 128 * c->keys_pad);      // tiled V^T [128][keys_pad]
+    c->add_buf("decoder_x", 64, 1024, 1024);                               // the decoder_* activations are fragment-tiled
+    c->add_buf("decoder_x_buf", 64, 1024, 1024);
+    c->add_buf("decoder_qkv", 64, 4096, 4096);                             // row-major
+    c->add_buf("decoder_Q", 8, 128 * 128, 128 * 128);
+    c->add_buf("decoder_attn", 64, 2048, 2048);
+    c->add_buf("decoder_hidden", 64, 2048, 2048);                          // 1536 columns used, the rest stays zero
+    const int64_t pmax = std::max(M * 1024, P * 2048) * 8;
+    c->add_buf("splitk_partial", 1, pmax, pmax, 4);
+    return 0;
+}
+
 // ------------------------------------------------------------------------------------------------
 // schedule
 // ------------------------------------------------------------------------------------------------
@@ -323,11 +436,11 @@ struct Sched {
     Sched(rtvla_ctx* c_, hipStream_t s_) : c(c_), s(s_), d(c_->d), pi05(c_->d.model == RTVLA_PI05) {}
 
     void gemm(const bf16_t* A, int lda, int a_rows, int M, const bf16_t* B0, const bf16_t* B1, int K, int N, int epi, GemmP extra, const char* what) {
-        const int bgroup = epi == EPI_GEGLU ? 4 : 8;
+        const int bgroup = (epi == EPI_GEGLU || epi == EPI_SWIGLU) ? 4 : 8;
         GemmP p = extra;
         p.A = A; p.lda = lda; p.a_rows = a_rows; p.M = M; p.B0 = B0; p.B1 = B1;
         p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.bgroup = bgroup;
-        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU, epi == EPI_PARTIAL, what);
+        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU || epi == EPI_SWIGLU, epi == EPI_PARTIAL, what);
         p.nsplit = tc.nsplit;
         if (epi == EPI_PARTIAL) {
             p.partial = c->B<float>("splitk_partial"); p.ldp = N; p.pstride = (size_t)M * N;
@@ -343,8 +456,9 @@ struct Sched {
     int last_split = 1;
 
     void reduce(int M, int N, const bf16_t* bias, const bf16_t* res, int ldr, bf16_t* x, int ldx, bf16_t* xn, int ldxn,
-                int norm, const bf16_t* nw, const bf16_t* nb, float eps, int nsplit, const char* what) {
+                int norm, const bf16_t* nw, const bf16_t* nb, float eps, int nsplit, const char* what, float* factor = nullptr) {
         ReduceP p{};
+        p.factor = factor;
         p.partial = c->B<float>("splitk_partial"); p.pstride = (size_t)M * N; p.ldp = N; p.nsplit = nsplit;
         p.bias = bias; p.res = res; p.ldr = ldr; p.x = x; p.ldx = ldx; p.xn = xn; p.ldxn = ldxn;
         p.M = M; p.N = N; p.norm = norm; p.nw = nw; p.nb = nb; p.eps = eps;
@@ -493,7 +607,199 @@ struct Sched {
         }
     }
 
+    // ---- DM0 (/root/reference/dm0_infer.py) ----
+    bf16_t* dK(int i) { return c->B("kv_K") + (size_t)i * 8 * c->keys_pad * 128; }
+    bf16_t* dVt(int i) { return c->B("kv_Vt") + (size_t)i * 8 * 128 * c->keys_pad; }
+    const float* WF(const char* n, size_t layer_elems, int layer) { return (const float*)c->tensors[c->tindex.at(n)].ptr + layer_elems * layer; }
+
+    // dm0_infer.py:695-712: patch embedding, class token, position embedding, ln_pre; then the first layer's LayerNorm
+    void dm0_vision_embed() {
+        const int n = d.num_views, M = n * DM0_SEQ;
+        if (c->want("im2col")) { launch_dm0_im2col_nchw(c->W("images"), c->B("vision_patches"), PATCH_LD, n, s); c->note(0, "im2col"); }
+        GemmP e{}; e.out = c->B("vision_conv1_buf"); e.ldo = 1024; e.bias = c->B("const_zeros");
+        gemm(c->B("vision_patches"), PATCH_LD, n * 2704, n * 2704, c->TW("t_vision_conv1_w_t"), nullptr, 588, 1024, EPI_BIAS, e, "patch embed");
+        if (c->want("class + pos + ln_pre")) {
+            launch_dm0_embed_ln(c->B("vision_conv1_buf"), c->W("vision_class_embedding"), c->W("vision_pos_emb"), c->W("vision_ln_pre_w"), c->W("vision_ln_pre_b"),
+                                c->B("vision_x_2d"), n, s);
+            c->note(0, "class + pos + ln_pre");
+        }
+        reduce(M, 1024, nullptr, c->B("vision_x_2d"), 1024, nullptr, 0, c->B("vision_x_norm"), 1024, NORM_LAYER, c->B("const_ones"), c->B("const_zeros"), 1e-5f, 0, "vit LN0");
+    }
+
+    // dm0_infer.py:718-736.  The LayerNorm scale and shift are folded into the weights; the rows are normalised by the reduce
+    // kernel (x_norm), which equals the reference's  rstd (x W' - mean colsum(W')) + b'  up to the rounding of x_norm.
+    void dm0_vision_layer(int i) {
+        const int n = d.num_views, M = n * DM0_SEQ;
+        GemmP e{}; e.bias_f32 = WF("vision_fused_qkv_b", 3072, i); e.rope = c->W("vision_rope"); e.seq = DM0_SEQ; e.seq_pad = DM0_SEQ_PAD;
+        e.q = c->B("vision_Q"); e.k = c->B("vision_K"); e.vt = c->B("vision_Vt");
+        gemm(c->B("vision_x_norm"), 1024, M, M, c->TW("t_vision_fused_qkv_w", i), nullptr, 1024, 3072, EPI_VIT_QKV_ROPE, e, "vit qkv");
+        AttnP a{};
+        a.q = c->B("vision_Q"); a.k = c->B("vision_K"); a.vt = c->B("vision_Vt"); a.ldvt = DM0_SEQ_PAD;
+        a.batch = n * 16; a.q_bstride = a.k_bstride = (size_t)DM0_SEQ_PAD * 64; a.vt_bstride = (size_t)64 * DM0_SEQ_PAD;
+        a.group = 1; a.rows = DM0_SEQ; a.keys = DM0_SEQ; a.scale = 0.125f; a.prefix_alloc = DM0_SEQ;
+        a.out = c->B("vision_attn"); a.ld_tok = 1024; a.batch_inner = 16; a.out_ostride = (size_t)DM0_SEQ * 1024; a.out_istride = 64;
+        if (c->want("vit attn")) c->note(launch_mqa_attention(a, ATTN_VIT64, s), "vit attn");
+        gemm(c->B("vision_attn"), 1024, M, M, c->TW("t_vision_out_proj_w", i), nullptr, 1024, 1024, EPI_PARTIAL, GemmP{}, "vit o");
+        reduce(M, 1024, c->W("vision_out_proj_b", 1024, i), c->B("vision_x_2d"), 1024, c->B("vision_x_2d"), 1024, c->B("vision_x_norm"), 1024,
+               NORM_LAYER, c->B("const_ones"), c->B("const_zeros"), 1e-5f, last_split, "vit o reduce");
+        GemmP u{}; u.out = c->B("vision_fc"); u.ldo = 4096; u.bias_f32 = WF("vision_fused_fc_b", 4096, i);
+        gemm(c->B("vision_x_norm"), 1024, M, M, c->TW("t_vision_fused_fc_w", i), nullptr, 1024, 4096, EPI_BIAS_GELU, u, "vit fc");
+        gemm(c->B("vision_fc"), 4096, M, M, c->TW("t_vision_proj_w", i), nullptr, 4096, 1024, EPI_PARTIAL, GemmP{}, "vit proj");
+        reduce(M, 1024, c->W("vision_proj_b", 1024, i), c->B("vision_x_2d"), 1024, c->B("vision_x_2d"), 1024, c->B("vision_x_norm"), 1024,
+               NORM_LAYER, c->B("const_ones"), c->B("const_zeros"), 1e-5f, last_split, "vit proj reduce");
+    }
+
+    // dm0_infer.py:738-756: drop the class token, two stride-2 3x3 convolutions, projector, token embeddings; then the RMS
+    // factor of the first prefix layer
+    void dm0_project() {
+        const int n = d.num_views, P = c->S_e, T = n * DM0_TOK;
+        if (c->want("im2col ds1")) { launch_dm0_im2col3x3(c->B("vision_x_2d"), DM0_SEQ, 1, 52, 52, 1024, c->B("vision_col1"), n, s); c->note(0, "im2col ds1"); }
+        GemmP e{}; e.out = c->B("vision_mm1"); e.ldo = 2048; e.bias = c->W("vision_ds1_b");
+        gemm(c->B("vision_col1"), 9216, n * 676, n * 676, c->TW("t_vision_ds1_w"), nullptr, 9216, 2048, EPI_BIAS, e, "ds1");
+        if (c->want("im2col ds2")) { launch_dm0_im2col3x3(c->B("vision_mm1"), 676, 0, 26, 26, 2048, c->B("vision_col2"), n, s); c->note(0, "im2col ds2"); }
+        GemmP f{}; f.out = c->B("vision_mm2"); f.ldo = 4096; f.bias = c->W("vision_ds2_b");
+        gemm(c->B("vision_col2"), 18432, T, T, c->TW("t_vision_ds2_w"), nullptr, 18432, 4096, EPI_BIAS, f, "ds2");
+        GemmP g{}; g.out = c->B("prefix_x"); g.ldo = 2048; g.bias = c->B("const_zeros");
+        gemm(c->B("vision_mm2"), 4096, T, T, c->TW("t_vision_projector_w_t"), nullptr, 4096, 2048, EPI_BIAS, g, "projector");
+        if (d.prompt_len > 0 && c->want("token embeddings")) {
+            launch_dm0_gather_rows(c->W("vision_embed_tokens_w"), (int)c->T("vision_embed_tokens_w").shape[0], (const int*)c->T("input_ids").ptr,
+                                   c->B("prefix_x") + (size_t)T * 2048, d.prompt_len, s);
+            c->note(0, "token embeddings");
+        }
+        reduce(P, 2048, nullptr, c->B("prefix_x"), 2048, nullptr, 0, nullptr, 0, NORM_RMS, nullptr, nullptr, 1e-6f, 0, "prefix factor0", c->B<float>("prefix_norm_factor"));
+    }
+
+    // dm0_infer.py:874-951
+    void dm0_prefix_layer(int i) {
+        const int P = c->S_e, kp = c->keys_pad;
+        const size_t qstride = (size_t)((2 * P + 31) / 32) * 32 * 128;
+        GemmP e{}; e.out = c->B("prefix_qkv"); e.ldo = 4096; e.bias = c->B("const_zeros");
+        gemm(c->B("prefix_x"), 2048, P, P, c->TW("t_llm_attn_qkv_w", i), nullptr, 2048, 4096, EPI_BIAS, e, "prefix qkv");
+        if (c->want("prefix qk-norm rope")) {
+            launch_dm0_qknorm_rope(c->B("prefix_qkv"), 4096, c->B<float>("prefix_norm_factor"), nullptr, c->W("llm_q_norm_w", 128, i), c->W("llm_k_norm_w", 128, i),
+                                   c->W("prefix_rope_weights"), c->B("prefix_Q"), qstride, dK(i), (size_t)kp * 128, dVt(i), (size_t)128 * kp, kp >> 5, 0, P, s);
+            c->note(0, "prefix qk-norm rope");
+        }
+        AttnP a{};
+        a.q = c->B("prefix_Q"); a.k = dK(i); a.vt = dVt(i); a.ldvt = kp;
+        a.batch = 8; a.q_bstride = qstride; a.k_bstride = (size_t)kp * 128; a.vt_bstride = (size_t)128 * kp;
+        a.group = 2; a.rows = 2 * P; a.keys = P; a.scale = 0.08838834764831845f; a.prefix_alloc = P; a.causal = 1;
+        a.out = c->B("prefix_attn"); a.ld_tok = 2048; a.batch_inner = 8; a.out_istride = 256;
+        if (c->want("prefix attn")) c->note(launch_mqa_attention(a, ATTN_GQA128_PREFIX, s), "prefix attn");
+        gemm(c->B("prefix_attn"), 2048, P, P, c->TW("t_llm_attn_o_w", i), nullptr, 2048, 2048, EPI_PARTIAL, GemmP{}, "prefix o");
+        reduce(P, 2048, nullptr, c->B("prefix_x"), 2048, c->B("prefix_x"), 2048, nullptr, 0, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix o reduce",
+               c->B<float>("prefix_norm_factor"));
+        GemmP g{}; g.out = c->B("prefix_hidden"); g.ldo = 6144; g.rowscale = c->B<float>("prefix_norm_factor");
+        gemm(c->B("prefix_x"), 2048, P, P, c->TW("t_llm_ffn_gate_w", i), c->TW("t_llm_ffn_up_w", i), 2048, 6144, EPI_SWIGLU, g, "prefix swiglu");
+        gemm(c->B("prefix_hidden"), 6144, P, P, c->TW("t_llm_ffn_down_w", i), nullptr, 6144, 2048, EPI_PARTIAL, GemmP{}, "prefix down");
+        reduce(P, 2048, nullptr, c->B("prefix_x"), 2048, c->B("prefix_x"), 2048, nullptr, 0, NORM_RMS, nullptr, nullptr, 1e-6f, last_split, "prefix down reduce",
+               c->B<float>("prefix_norm_factor"));
+    }
+
+    // dm0_infer.py:763-780
+    void dm0_step_begin(int t) {
+        const int ch = d.chunk_size;
+        if (c->want("action in")) {
+            launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_fused_in_proj_w"), c->W("decoder_action_fused_time_biases", 1024, t % 10),
+                                c->B("decoder_x_buf"), 1024, ch, 32, 1024, 1, 1, 0, s);
+            c->note(0, "action in");
+        }
+        SkinnyP e = tiled_io(); e.out = c->B("decoder_x"); e.ldo = 1024; e.bias = c->W("decoder_action_mlp_b");
+        skinny(c->B("decoder_x_buf"), 1024, ch, c->TW("t_decoder_action_mlp_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS, e, "action mlp");
+    }
+
+    // dm0_infer.py:782-851
+    void dm0_suffix_layer(int t, int i) {
+        const int ch = d.chunk_size, P = c->S_e, kp = c->keys_pad;
+        SkinnyP q{}; q.a_tiled = 1; q.out = c->B("decoder_qkv"); q.ldo = 4096; q.bias = c->B("const_zeros");
+        skinny(c->B("decoder_x"), 1024, ch, c->TW("t_decoder_attn_qkv_w", i), nullptr, 1024, 4096, SN_NONE, nullptr, SK_BIAS, q, "suffix qkv");
+        if (c->want("suffix qk-norm rope")) {
+            launch_dm0_qknorm_rope(c->B("decoder_qkv"), 4096, nullptr, c->B("decoder_x"), c->W("decoder_q_norm_w", 128, i), c->W("decoder_k_norm_w", 128, i),
+                                   c->W("decoder_rope_weights"), c->B("decoder_Q"), (size_t)128 * 128, dK(i), (size_t)kp * 128, dVt(i), (size_t)128 * kp, kp >> 5, P, ch, s);
+            c->note(0, "suffix qk-norm rope");
+        }
+        AttnP a{};
+        a.q = c->B("decoder_Q"); a.k = dK(i); a.vt = dVt(i); a.ldvt = kp;
+        a.batch = 8; a.q_bstride = (size_t)128 * 128; a.k_bstride = (size_t)kp * 128; a.vt_bstride = (size_t)128 * kp;
+        a.group = 2; a.rows = 2 * ch; a.keys = P + ch; a.scale = 0.08838834764831845f; a.prefix_alloc = P + ch;
+        a.out = c->B("decoder_attn"); a.out_tiled = 1; a.out_bcol = 256; a.out_cols32 = 64;
+        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_GQA128_SUFFIX, s), "suffix attn");
+        SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024;
+        skinny(c->B("decoder_attn"), 2048, ch, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
+        SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 2048; g.factor_f32 = 1;
+        skinny(c->B("decoder_x"), 1024, ch, c->TW("t_decoder_ffn_gate_w", i), c->TW("t_decoder_ffn_up_w", i), 1024, 1536, SN_RMS, nullptr, SK_SWIGLU, g, "suffix swiglu");
+        SkinnyP dn = tiled_io(); dn.out = c->B("decoder_x"); dn.ldo = 1024;
+        skinny(c->B("decoder_hidden"), 2048, ch, c->TW("t_decoder_ffn_down_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, dn, "suffix down");
+    }
+
+    // dm0_infer.py:863-872, :99-120
+    void dm0_step_end(int t) {
+        SkinnyP e{}; e.a_tiled = 1; e.out = c->W("diffusion_noise"); e.ldo = 32; e.bias = c->W("decoder_action_fused_out_proj_b"); e.factor_f32 = 1;
+        skinny(c->B("decoder_x"), 1024, d.chunk_size, c->TW("t_decoder_out_proj_w"), nullptr, 1024, 32, SN_RMS, nullptr, SK_RES, e, "euler");
+    }
+
+    void dm0_prepare(bool tiles_loaded) {
+        const int V = d.vision_layers, L = d.llm_layers;
+        launch_fill_zero(c->ws + c->act_begin, c->ws_bytes - c->act_begin, s);
+        launch_fill_bf16(c->B("const_ones"), 1024, 1.0f, s);
+        if (tiles_loaded) return;
+        auto tile = [&](const char* src, const char* dst, int K, int N, int layers) {
+            for (int i = 0; i < layers; ++i) launch_pretile(c->W(src, (size_t)K * N, i), K, N, c->TW(dst, i), c->tgroup.at(dst), c->twide.at(dst), s);
+        };
+        tile("vision_conv1_w_t", "t_vision_conv1_w_t", 588, 1024, 1);
+        tile("vision_fused_qkv_w", "t_vision_fused_qkv_w", 1024, 3072, V);
+        tile("vision_out_proj_w", "t_vision_out_proj_w", 1024, 1024, V);
+        tile("vision_fused_fc_w", "t_vision_fused_fc_w", 1024, 4096, V);
+        tile("vision_proj_w", "t_vision_proj_w", 4096, 1024, V);
+        tile("vision_ds1_w", "t_vision_ds1_w", 9216, 2048, 1);
+        tile("vision_ds2_w", "t_vision_ds2_w", 18432, 4096, 1);
+        tile("vision_projector_w_t", "t_vision_projector_w_t", 4096, 2048, 1);
+        tile("llm_attn_qkv_w", "t_llm_attn_qkv_w", 2048, 4096, L);
+        tile("llm_attn_o_w", "t_llm_attn_o_w", 2048, 2048, L);
+        tile("llm_ffn_gate_w", "t_llm_ffn_gate_w", 2048, 6144, L);
+        tile("llm_ffn_up_w", "t_llm_ffn_up_w", 2048, 6144, L);
+        tile("llm_ffn_down_w", "t_llm_ffn_down_w", 6144, 2048, L);
+        tile("decoder_attn_qkv_w", "t_decoder_attn_qkv_w", 1024, 4096, L);
+        tile("decoder_attn_o_w", "t_decoder_attn_o_w", 2048, 1024, L);
+        tile("decoder_ffn_gate_w", "t_decoder_ffn_gate_w", 1024, 1536, L);
+        tile("decoder_ffn_up_w", "t_decoder_ffn_up_w", 1024, 1536, L);
+        for (int i = 0; i < L; ++i)       // K = 1536 rows of the checkpoint, laid out for K = 2048 with zero rows behind
+            launch_pretile_padded(c->W("decoder_ffn_down_w", (size_t)1536 * 1024, i), 1536, 2048, 1024, c->TW("t_decoder_ffn_down_w", i), s);
+        tile("decoder_action_mlp_w", "t_decoder_action_mlp_w", 1024, 1024, 1);
+        tile("decoder_action_fused_out_proj_w", "t_decoder_out_proj_w", 1024, 32, 1);
+    }
+
+    int dm0_stage(int st, int layer, int step) {
+        switch (st) {
+            case RTVLA_STAGE_VISION_EMBED: dm0_vision_embed(); break;
+            case RTVLA_STAGE_VISION_LAYER: if (layer < 0 || layer >= d.vision_layers) return RTVLA_ERR_ARG; dm0_vision_layer(layer); break;
+            case RTVLA_STAGE_PROJECT: dm0_project(); break;
+            case RTVLA_STAGE_PREFIX_LAYER: if (layer < 0 || layer >= d.llm_layers) return RTVLA_ERR_ARG; dm0_prefix_layer(layer); break;
+            case RTVLA_STAGE_SUFFIX_INIT: break;
+            case RTVLA_STAGE_SUFFIX_STEP_BEGIN: if (step < 0 || step >= d.num_steps) return RTVLA_ERR_ARG; dm0_step_begin(step); break;
+            case RTVLA_STAGE_SUFFIX_LAYER:
+                if (layer < 0 || layer >= d.llm_layers || step < 0 || step >= d.num_steps) return RTVLA_ERR_ARG;
+                dm0_suffix_layer(step, layer); break;
+            case RTVLA_STAGE_SUFFIX_STEP_END: if (step < 0 || step >= d.num_steps) return RTVLA_ERR_ARG; dm0_step_end(step); break;
+            default: return RTVLA_ERR_ARG;
+        }
+        return 0;
+    }
+
+    void dm0_forward() {
+        dm0_vision_embed();
+        for (int i = 0; i < d.vision_layers; ++i) dm0_vision_layer(i);
+        dm0_project();
+        for (int i = 0; i < d.llm_layers; ++i) dm0_prefix_layer(i);
+        for (int t = 0; t < d.num_steps; ++t) {
+            dm0_step_begin(t);
+            for (int i = 0; i < d.llm_layers; ++i) dm0_suffix_layer(t, i);
+            dm0_step_end(t);
+        }
+    }
+
     int stage(int st, int layer, int step) {
+        if (d.model == RTVLA_DM0) return dm0_stage(st, layer, step);
         switch (st) {
             case RTVLA_STAGE_VISION_EMBED: vision_embed(); break;
             case RTVLA_STAGE_VISION_LAYER: if (layer < 0 || layer >= d.vision_layers) return RTVLA_ERR_ARG; vision_layer(layer); break;
@@ -511,6 +817,7 @@ struct Sched {
     }
 
     void forward() {
+        if (d.model == RTVLA_DM0) { dm0_forward(); return; }
         vision_embed();
         for (int i = 0; i < d.vision_layers; ++i) vision_layer(i);
         project();
@@ -526,6 +833,7 @@ struct Sched {
     // one-time device work.  With `tiles_loaded` the re-tiled weights (the first rtvla_tiled_bytes of the workspace) were
     // filled in by the caller from a copy saved after an earlier prepare, and only the rest is done.
     void prepare(bool tiles_loaded) {
+        if (d.model == RTVLA_DM0) { dm0_prepare(tiles_loaded); return; }
         const int V = d.vision_layers, L = d.llm_layers;
         launch_fill_zero(c->ws + c->act_begin, c->ws_bytes - c->act_begin, s);
         auto tile = [&](const char* src, const char* dst, int K, int N, int layers) {
@@ -613,22 +921,22 @@ int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out) {
     if (!dims || !out) return RTVLA_ERR_ARG;
     *out = nullptr;
     const rtvla_dims& d = *dims;
-    if (d.model != RTVLA_PI0 && d.model != RTVLA_PI05) return RTVLA_ERR_ARG;
+    if (d.model != RTVLA_PI0 && d.model != RTVLA_PI05 && d.model != RTVLA_DM0) return RTVLA_ERR_ARG;
     if (d.num_views < 1 || d.num_views > 4 || d.prompt_len < 0 || d.chunk_size < 1 || d.num_steps < 1) return RTVLA_ERR_ARG;
     if (d.vision_layers < 1 || d.llm_layers < 1) return RTVLA_ERR_ARG;
     const int S_d = d.chunk_size + (d.model == RTVLA_PI0 ? 1 : 0);
     if (S_d > 64) return RTVLA_ERR_LIMIT;
-    if (d.model == RTVLA_PI05 && d.num_steps > 10) return RTVLA_ERR_LIMIT;      // decoder_time_embeds has 10 rows
+    if (d.model != RTVLA_PI0 && d.num_steps > 10) return RTVLA_ERR_LIMIT;       // the per-step time tables have 10 rows
     if (d.prompt_len > 4096) return RTVLA_ERR_LIMIT;
     rtvla_ctx* c = new (std::nothrow) rtvla_ctx();
     if (!c) return RTVLA_ERR_ARG;
     c->d = d;
-    c->S_v = 256 * d.num_views;
+    c->S_v = (d.model == RTVLA_DM0 ? DM0_TOK : 256) * d.num_views;
     c->S_e = c->S_v + d.prompt_len;
     c->S_d = S_d;
     c->keys = c->S_e + c->S_d;
     c->keys_pad = ((c->keys + 63) / 64) * 64;
-    build_tables(c);
+    if (d.model == RTVLA_DM0) build_tables_dm0(c); else build_tables(c);
     *out = c;
     return RTVLA_OK;
 }
@@ -663,7 +971,7 @@ int rtvla_bind(rtvla_ctx* c, const char* name, void* ptr, size_t bytes) {
     auto it = c->tindex.find(name);
     if (it == c->tindex.end()) return c->fail(RTVLA_ERR_NAME, std::string("unknown tensor: ") + name);
     Tensor& t = c->tensors[it->second];
-    if (t.name == "embedding_weight" && bytes > 0 && bytes % 4096 == 0) t.shape[0] = (int64_t)(bytes / 4096);
+    if ((t.name == "embedding_weight" || t.name == "vision_embed_tokens_w") && bytes > 0 && bytes % 4096 == 0) t.shape[0] = (int64_t)(bytes / 4096);
     if (bytes != t.bytes()) return c->fail(RTVLA_ERR_SIZE, std::string("size mismatch for ") + name + ": got " + std::to_string(bytes) + ", want " + std::to_string(t.bytes()));
     if (!ptr && bytes) return c->fail(RTVLA_ERR_ARG, std::string("null pointer for ") + name);
     if (((uintptr_t)ptr & 15) != 0) return c->fail(RTVLA_ERR_ARG, std::string("pointer not 16-byte aligned: ") + name);

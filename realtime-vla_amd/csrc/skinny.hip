@@ -23,7 +23,7 @@ template <int NCH, int NORM, int EPI, int SK_MTS>
 __global__ __launch_bounds__(SK_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void skinny_kernel(SkinnyP p) {
     constexpr int KBW = NCH * SK_CH;
-    constexpr bool DUAL = (EPI == SK_GEGLU);
+    constexpr bool DUAL = (EPI == SK_GEGLU || EPI == SK_SWIGLU);
     constexpr int NB = DUAL ? 2 : 1;
     static_assert(NORM == SN_NONE || NCH == 1, "the fused norm needs the whole K slice in registers");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -169,7 +169,8 @@ void skinny_kernel(SkinnyP p) {
         float t = 0.f;
 #pragma unroll
         for (int ww = 0; ww < SK_WAVES; ++ww) t += ssq[ww * 64 + mt * 16 + r];
-        const float f = round_bf16(rsqrtf(t / (float)p.K + p.eps));      // the reference keeps the factor in bf16
+        float f = rsqrtf(t / (float)p.K + p.eps);
+        if (!p.factor_f32) f = round_bf16(f);                            // the Pi0 reference keeps the factor in bf16, DM0 in fp32
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) v[nb] *= f;
     }
@@ -193,6 +194,8 @@ void skinny_kernel(SkinnyP p) {
     } else if constexpr (EPI == SK_GEGLU) {
         store4(optr,
                pack4(gelu_tanh(v[0][0]) * v[1][0], gelu_tanh(v[0][1]) * v[1][1], gelu_tanh(v[0][2]) * v[1][2], gelu_tanh(v[0][3]) * v[1][3]));
+    } else if constexpr (EPI == SK_SWIGLU) {
+        store4(optr, pack4(siluf(v[0][0]) * v[1][0], siluf(v[0][1]) * v[1][1], siluf(v[0][2]) * v[1][2], siluf(v[0][3]) * v[1][3]));
     } else if constexpr (EPI == SK_QKV_ROPE) {
         f32x4 o = v[0];
         if (n0 < 2304) {
@@ -213,7 +216,7 @@ void skinny_kernel(SkinnyP p) {
 
 template <int NCH, int NORM, int EPI, int SK_MTS>
 int launch_inst(const SkinnyP& p, hipStream_t s) {
-    constexpr int NB = (EPI == SK_GEGLU) ? 2 : 1;
+    constexpr int NB = (EPI == SK_GEGLU || EPI == SK_SWIGLU) ? 2 : 1;
     const size_t smem = (size_t)SK_WAVES * NB * SK_MTS * 64 * 16 + (size_t)SK_WAVES * 64 * 4;
     auto kern = skinny_kernel<NCH, NORM, EPI, SK_MTS>;
     if (smem > 65536) {
@@ -245,6 +248,7 @@ int launch_skinny(const SkinnyP& p, int epi, hipStream_t s) {
     SK_CASE(1, SN_ADARMS, SK_QKV_ROPE, 4);
     SK_CASE(1, SN_RMS, SK_GEGLU, 4);
     SK_CASE(1, SN_ADARMS, SK_GEGLU, 4);
+    SK_CASE(1, SN_RMS, SK_SWIGLU, 4);
     SK_CASE(1, SN_NONE, SK_BIAS, 4);
     SK_CASE(1, SN_NONE, SK_BIAS_SILU, 4);
     SK_CASE(1, SN_RMS, SK_RES, 4);

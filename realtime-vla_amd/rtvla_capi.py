@@ -9,7 +9,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RTVLA_LIBRARY") or os.path.join(HERE, "librtvla.so")   # override: an alternative build of the same ABI
 
-PI0, PI05 = 0, 1
+PI0, PI05, DM0 = 0, 1, 2
 
 STAGE_VISION_EMBED = 0
 STAGE_VISION_LAYER = 1

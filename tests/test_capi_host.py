@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
 
 
 def test_create_validates_dimensions(lib):
-    for bad in [(capi.PI0, 0, 0, 50), (capi.PI0, 5, 0, 50), (capi.PI0, 1, -1, 50), (capi.PI0, 1, 0, 0), (2, 1, 0, 50)]:
+    for bad in [(capi.PI0, 0, 0, 50), (capi.PI0, 5, 0, 50), (capi.PI0, 1, -1, 50), (capi.PI0, 1, 0, 0), (3, 1, 0, 50), (capi.DM0, 0, 10, 50), (capi.DM0, 5, 10, 50)]:
         with pytest.raises(capi.RtvlaError):
             capi.Context(*bad)
     with pytest.raises(capi.RtvlaError) as e:
@@ -57,6 +57,24 @@ def test_tensor_table_matches_the_reference_layout(lib):
     assert t5["decoder_pre_attn_norm_mod_w"] == (2, (18, 1024, 3072), True)
     assert t5["decoder_rope_weights"] == (2, (50, 256), False)
     assert "observation_state_normalized" not in t5 and "decoder_state_in_proj_w" not in t5
+
+
+def test_dm0_tensor_table(lib):
+    """dm0_infer.py:986-1026 (weights), 754 (token ids)."""
+    c = capi.Context(capi.DM0, 3, 100, 50, 10, 23, 28)
+    t = {n: (e, s, w) for n, e, s, w, _ in c.tensors()}
+    assert t["images"] == (2, (3, 3, 728, 728), False)
+    assert t["input_ids"] == (4, (100,), False)
+    assert t["diffusion_noise"] == (2, (50, 32), False)
+    assert t["prefix_rope_weights"] == (2, (3 * 169 + 100, 128), False)
+    assert t["decoder_rope_weights"] == (2, (50, 128), False)
+    assert t["vision_fused_qkv_w"] == (2, (23, 1024, 3072), True)
+    assert t["vision_qkv_col_sum"] == (4, (23, 3072), True)          # fp32, as the reference keeps them
+    assert t["llm_attn_qkv_w"] == (2, (28, 2048, 4096), True)
+    assert t["decoder_attn_qkv_w"] == (2, (28, 1024, 4096), True)
+    assert t["vision_ds2_w"] == (2, (3, 3, 2048, 4096), True)
+    assert 0 < c.workspace_bytes() < 6 << 30
+    c.close()
 
 
 def test_bind_errors_are_status_codes(lib):

@@ -284,3 +284,14 @@ def test_dm0_language_tokens_follow_the_image_tokens(ck):
     img, ids, noise = syn.dm0_observation(52, 1, max_lang_len=4, vocab=64)
     x = dm0.vision_forward(ck, img, ids, ID)
     assert x.shape == (169 + 4, 2048) and torch.equal(x[169:], ck["vision_embed_tokens_w"][ids].float())
+
+
+def test_host_side_rope_pair_table_matches_the_oracle_tables():
+    """The product's table (realtime-vla_amd/dm0_infer.py) holds one (cos, sin) per rotation pair; the reference's 64 angles
+    repeat each frequency for both elements of a pair."""
+    from dm0_infer import vision_rope_pairs
+    tab = vision_rope_pairs("cpu").float()
+    cos, sin = dm0.vision_rope_table()
+    assert tab.shape == (2705, 64)
+    assert torch.equal(tab[:, 0::2], cos[:, 0::2]) and torch.equal(tab[:, 0::2], cos[:, 1::2])
+    assert torch.equal(tab[:, 1::2], sin[:, 0::2]) and torch.equal(tab[:, 1::2], sin[:, 1::2])
