@@ -1,6 +1,6 @@
 """Latency benchmark of the Pi0 / Pi05 single-observation forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config headline|c1|c2|c3|c4|c5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config headline|c1|c2|c3|c4|c5|dm0] [--no-cpu]
 
 A "step" is one forward (vision encoder + prefix pass + 10 flow steps) on synthetic inputs that are
 already resident in HBM.  Prints ONE JSON line: p50 latency (ms) as `value`, the live roofline of the
@@ -24,6 +24,7 @@ CONFIGS = {
     "c3": ("pi0", 3, 0, 63, 0, "Pi0, 3 views, empty prompt, chunk 63, 10 flow steps"),
     "c4": ("pi05", 3, 20, 50, 32, "Pi05, 3 views, 20 prompt + 32 state tokens, chunk 50, 10 flow steps"),
     "c5": ("pi0", 3, 200, 50, 0, "Pi0, 3 views, 200-token prompt (968-token prefix), chunk 50, 10 flow steps"),
+    "dm0": ("dm0", 3, 100, 50, 0, "DM0, 3 images of 728x728, 100 language tokens, chunk 50, 10 flow steps"),
 }
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
@@ -111,6 +112,94 @@ def bench_transforms(args, dev):
     print(json.dumps(result))
 
 
+def bench_dm0(args, dev, desc, views, lang, chunk):
+    """The reference's third model at its own benchmark shape (/root/reference/benchmark.py:61-62, README.md:35)."""
+    import torch
+    import synthetic as syn
+    import rtvla_capi as capi
+    from dm0_infer import DM0Inference
+    seed = 1234
+    ck = syn.dm0_checkpoint(seed, dev)
+    img, ids, noise = syn.dm0_observation(seed, views, dev, max_lang_len=lang)
+    model = DM0Inference(ck, num_images=views, max_lang_len=lang)
+    ctx, stream = model._engine.ctx, torch.cuda.current_stream().cuda_stream
+    lib_version = capi.load().rtvla_version()
+    draws = [syn.dm0_observation(seed, views, dev, max_lang_len=lang, draw=i)[2] for i in range(16)]
+    for i in range(args.warmup):
+        model.forward(img, ids, draws[i % 16])
+    torch.cuda.synchronize()
+    times = []
+    t_all0 = time.perf_counter()
+    for i in range(args.steps):
+        torch.cuda.synchronize(); t0 = time.perf_counter()
+        model.forward(img, ids, draws[i % 16])
+        torch.cuda.synchronize(); times.append((time.perf_counter() - t0) * 1e3)
+    t_all = (time.perf_counter() - t_all0) * 1e3
+    st = sorted(times)
+    p50, p99 = st[len(st) // 2], st[min(len(st) - 1, int(0.99 * len(st)))]
+    # every launch of one ViT / prefix / action-expert layer (weights cold: cycled over the layers)
+    launches = {}
+    for label, stage in (("vit", capi.STAGE_VISION_LAYER), ("prefix", capi.STAGE_PREFIX_LAYER), ("action", capi.STAGE_SUFFIX_LAYER)):
+        rows = []
+        for idx in range(16):
+            r = ctx.time_launch(stage, -1, 0, idx, 3, stream)
+            if r is None:
+                break
+            rows.append((r[1], round(r[0] * 1e3, 2)))
+        launches[label] = {"launches_us": rows, "layer_us": round(ctx.time_stage(stage, -1, 0, 3, stream) * 1e3, 2)}
+    stages = {name: round(ctx.time_stage(stage, 0, 0, 5, stream) * 1e3, 2) for name, stage in
+              (("patch_embed_us", capi.STAGE_VISION_EMBED), ("downsample_project_us", capi.STAGE_PROJECT))}
+    M, P = views * 2705, views * 169 + lang
+    fc = next((r for r in launches["vit"]["launches_us"] if "fc" in r[0]), None)
+    fc_flop = 2.0 * M * 1024 * 4096
+    roofline = None
+    if fc:
+        tf = fc_flop / (fc[1] * 1e-6) / 1e12
+        roofline = {"bound": "mfma", "kernel": "ViT MLP up-projection with folded LayerNorm and GELU (gemm_mfma_kernel), M=%d K=1024 N=4096" % M,
+                    "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS, 4),
+                    "launch_ms": round(fc[1] / 1e3, 4), "traffic": None, "kernel_variant": fc[0],
+                    "algorithmic_bytes": 2.0 * (M * 1024 + 1024 * 4096 + M * 4096)}
+    d_l = 1024 * 4096 + 2048 * 1024 + 3 * 1024 * 1536
+    layer_bytes = 2.0 * d_l + 2.0 * (P + chunk) * 8 * 128 * 2
+    hbm = layer_bytes / (launches["action"]["layer_us"] * 1e-6) / 1e9
+    roofline_hbm = {"bound": "hbm", "kernel": "one DM0 action-expert layer", "achieved": round(hbm, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(hbm / HBM_PEAK_GBS, 4), "launch_ms": round(launches["action"]["layer_us"] / 1e3, 4), "traffic": None,
+                    "algorithmic_bytes": layer_bytes}
+    v_l = 1024 * 3072 + 1024 * 1024 + 2 * 1024 * 4096
+    e_l = 2048 * 4096 + 2048 * 2048 + 3 * 2048 * 6144
+    f_vis = 2.0 * M * (588 * 1024 + 23 * v_l) + 23 * views * 16 * 4.0 * 2705 * 2705 * 64 \
+        + 2.0 * views * (676 * 9216 * 2048 + 169 * 18432 * 4096 + 169 * 4096 * 2048)
+    f_pre = 2.0 * P * 28 * e_l + 28 * 16 * 4.0 * P * P * 128 / 2
+    b_dec = 10 * 28 * layer_bytes
+    ideal_ms = ((f_vis + f_pre) / (MFMA_PEAK_TFLOPS * 1e12) + b_dec / (HBM_PEAK_GBS * 1e9)) * 1e3
+    result = {"metric": "p50 ms per DM0 forward (%d images, chunk %d, 10 steps); %% roofline" % (views, chunk),
+              "value": round(p50, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "ms_per_step": round(t_all / args.steps, 4), "p99_ms": round(p99, 4), "higher_is_better": False, "scaling": "weak",
+              "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+              "config": {"workload": desc, "config_id": "dm0", "vit_tokens": M, "prefix_len": P, "graph_launches": model._engine.graph_launches,
+                         "weights": "seeded N(0, 0.02^2) bf16, random norm weights", "rtvla_version": lib_version},
+              "roofline": roofline, "roofline_hbm": roofline_hbm, "layers": launches, "stages": stages,
+              "forward_roofline_frac": round(ideal_ms / p50, 4), "forward_ideal_ms": round(ideal_ms, 4),
+              "reference_published": {"value_ms": 55.8, "hardware": "RTX 5090, Triton", "source": "README.md:35"}}
+    if not args.no_cpu:
+        from oracle import dm0 as od                      # the checker, timed as a baseline only
+        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or os.cpu_count()
+        torch.set_num_threads(cores)
+        ckc = {k: v.cpu() for k, v in ck.items()}
+        cpu_times = []
+        for it in range(1 + args.cpu_runs):
+            t0 = time.perf_counter()
+            ref = od.forward(ckc, img.cpu(), ids.cpu(), draws[0].cpu())
+            if it:
+                cpu_times.append((time.perf_counter() - t0) * 1e3)
+        out = model.forward(img, ids, draws[0]).float().cpu()
+        result["cpu_baseline"] = {"value": round(sorted(cpu_times)[len(cpu_times) // 2], 1), "unit": "ms", "cores": cores, "kind": "port",
+                                  "sample": "median of %d forwards of the same workload after 1 warm-up, PyTorch CPU eager oracle" % args.cpu_runs,
+                                  "runs_ms": [round(t, 1) for t in cpu_times]}
+        result["action_mae_vs_oracle"] = round((out - ref).abs().mean().item(), 5)
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,6 +233,8 @@ def main():
     seed = 1234
     if args.transforms:
         return bench_transforms(args, dev)
+    if model_name == "dm0":
+        return bench_dm0(args, dev, desc, views, prompt, chunk)
     if model_name == "pi0":
         from pi0_infer import Pi0Inference
         ck = syn.pi0_checkpoint(seed, prompt, device=dev)

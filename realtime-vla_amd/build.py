@@ -8,7 +8,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librtvla.so")
-SOURCES = ["gemm.hip", "skinny.hip", "attention.hip", "misc.hip", "dm0.hip", "rtvla.hip", "transforms.hip"]
+SOURCES = ["gemm.hip", "skinny.hip", "attention.hip", "misc.hip", "dm0.hip", "flash.hip", "rtvla.hip", "transforms.hip"]
 # bit-exact parity with host arithmetic (Pillow, numpy): no fused multiply-adds in these files
 EXTRA = {"transforms.hip": ["-ffp-contract=off"]}
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-unused-value",

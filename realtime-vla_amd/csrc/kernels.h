@@ -147,6 +147,8 @@ struct AttnP {
 // prefix and suffix; DM0 ViT (HD 64)
 enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1, ATTN_GQA128_PREFIX, ATTN_GQA128_SUFFIX, ATTN_VIT64 };
 int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s);
+// long sequences on both sides (csrc/flash.hip): 128 query rows per workgroup, K / V^T tiles shared through LDS; hd = 64
+int launch_flash_attention(const AttnP& p, int hd, hipStream_t s);
 // SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major
 void launch_vision_attention(const bf16_t* q, const bf16_t* k, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);
 

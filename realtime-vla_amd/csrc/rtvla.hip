@@ -638,7 +638,7 @@ struct Sched {
         a.batch = n * 16; a.q_bstride = a.k_bstride = (size_t)DM0_SEQ_PAD * 64; a.vt_bstride = (size_t)64 * DM0_SEQ_PAD;
         a.group = 1; a.rows = DM0_SEQ; a.keys = DM0_SEQ; a.scale = 0.125f; a.prefix_alloc = DM0_SEQ;
         a.out = c->B("vision_attn"); a.ld_tok = 1024; a.batch_inner = 16; a.out_ostride = (size_t)DM0_SEQ * 1024; a.out_istride = 64;
-        if (c->want("vit attn")) c->note(launch_mqa_attention(a, ATTN_VIT64, s), "vit attn");
+        if (c->want("vit attn")) c->note(launch_flash_attention(a, 64, s), "vit attn");
         gemm(c->B("vision_attn"), 1024, M, M, c->TW("t_vision_out_proj_w", i), nullptr, 1024, 1024, EPI_PARTIAL, GemmP{}, "vit o");
         reduce(M, 1024, c->W("vision_out_proj_b", 1024, i), c->B("vision_x_2d"), 1024, c->B("vision_x_2d"), 1024, c->B("vision_x_norm"), 1024,
                NORM_LAYER, c->B("const_ones"), c->B("const_zeros"), 1e-5f, last_split, "vit o reduce");
