@@ -212,7 +212,7 @@ void mqa_kernel(AttnP p) {
     }
     // partial record of one (row block, split): MQ x { O [DT][64] f32x4 | max [16] | sum [16] }
     constexpr int REC = DT * 64 * 4 + 32;
-    float* const mine = p.partial + ((size_t)rowblk * nsplit + split) * (MQ * REC);
+    float* const mine = p.partial + (((size_t)batch * p.row_blocks + rowblk) * nsplit + split) * (MQ * REC);
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         __syncthreads();                       // ls written / previous obuf round consumed
@@ -238,16 +238,18 @@ void mqa_kernel(AttnP p) {
     }
 }
 
-// Combine the key-split partials of mqa_kernel: one wave per (row block, 16-wide d tile), 4 waves per workgroup.
-// All loads of a wave are independent, so the kernel is one memory round trip long.
-template <int MQ, int NS>
+// Combine the key-split partials of mqa_kernel: one wave per (row block, 16-wide d tile), 4 waves per workgroup, K/V heads
+// along blockIdx.y.  All loads of a wave are independent, so the kernel is one memory round trip long.
+template <int MQ, int NS, int HD>
 __global__ __launch_bounds__(256)
 void attn_merge_kernel(AttnP p, int nsplit) {
-    constexpr int REC = 16 * 64 * 4 + 32;
+    constexpr int DT = HD / 16;
+    constexpr int REC = DT * 64 * 4 + 32;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
-    const int rb = blockIdx.x >> 2, dt = (blockIdx.x & 3) * 4 + w;
-    const float* const all = p.partial + (size_t)rb * nsplit * (MQ * REC);
+    const int batch = blockIdx.y;
+    const int rb = blockIdx.x / (DT / 4), dt = (blockIdx.x % (DT / 4)) * 4 + w;
+    const float* const all = p.partial + ((size_t)batch * p.row_blocks + rb) * nsplit * (MQ * REC);
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
         float ms[NS], ls[NS];
@@ -255,7 +257,7 @@ void attn_merge_kernel(AttnP p, int nsplit) {
 #pragma unroll
         for (int sp = 0; sp < NS; ++sp) {
             const float* rec = all + (size_t)min(sp, nsplit - 1) * (MQ * REC) + mq * REC;
-            ms[sp] = rec[4096 + r]; ls[sp] = rec[4112 + r];
+            ms[sp] = rec[DT * 256 + r]; ls[sp] = rec[DT * 256 + 16 + r];
             os[sp] = *(const f32x4*)(rec + (dt * 64 + lane) * 4);
         }
         float mg = NEG_BIG;
@@ -273,7 +275,7 @@ void attn_merge_kernel(AttnP p, int nsplit) {
         const int row = (rb * MQ + mq) * 16 + r;
         if (row < p.rows) {
             const int d = dt * 16 + 4 * g;
-            store4(attn_out_ptr(p, 0, row, d, 256), pack4(t * inv));
+            store4(attn_out_ptr(p, batch, row, d, HD), pack4(t * inv));
         }
     }
 }
@@ -374,13 +376,14 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
     p.kb_per_split = (nkb + want - 1) / want;
     const int nsplit = (nkb + p.kb_per_split - 1) / p.kb_per_split;
     if (nsplit > 1) {
-        if (!p.partial || nsplit > 16 || HD != 256 || p.batch > 1) return 1;      // the key split over workgroups exists for the Gemma suffix pass only
-        if ((size_t)blocks * nsplit * MQ * (16 * 64 * 4 + 32) > p.partial_floats) return 3;
+        if (!p.partial || nsplit > 16 || HD < 64 || p.causal) return 1;           // the key split over workgroups exists for the suffix passes
+        if ((size_t)p.batch * blocks * nsplit * MQ * ((HD / 16) * 64 * 4 + 32) > p.partial_floats) return 3;
     }
     p.nsplit_eff = nsplit;
+    p.row_blocks = blocks;
     hipLaunchKernelGGL(kern, dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(WAVES * 64), smem, s, p);
-    if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
-    else if (nsplit > 1) hipLaunchKernelGGL((attn_merge_kernel<MQ, 8>), dim3(blocks * 4), dim3(256), 0, s, p, nsplit);
+    if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16, HD>), dim3(blocks * (HD / 64), p.batch), dim3(256), 0, s, p, nsplit);
+    else if (nsplit > 1) hipLaunchKernelGGL((attn_merge_kernel<MQ, 8, HD>), dim3(blocks * (HD / 64), p.batch), dim3(256), 0, s, p, nsplit);
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 

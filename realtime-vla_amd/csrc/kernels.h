@@ -140,7 +140,7 @@ struct AttnP {
     int prefix_alloc; const int* valid_len; int state_rows;
     // key split over workgroups (nsplit > 1, at most 16): fp32 partial records, combined by a second launch
     int nsplit; float* partial; size_t partial_floats;
-    int kb_per_split, nsplit_eff;    // filled by the launcher
+    int kb_per_split, nsplit_eff, row_blocks;    // filled by the launcher
     RTVLA_KO_FIELD
 };
 // Gemma (HD 256): many rows, two row tiles per workgroup / few rows, one row tile and a key split; DM0 grouped-query (HD 128)

@@ -422,6 +422,7 @@ int build_tables_dm0(rtvla_ctx* c) {
     c->add_buf("decoder_hidden", 64, 2048, 2048);                          // 1536 columns used, the rest stays zero
     const int64_t pmax = std::max(M * 1024, P * 2048) * 8;
     c->add_buf("splitk_partial", 1, pmax, pmax, 4);
+    c->add_buf("attn_partial", 1, ATTN_PARTIAL_FLOATS, ATTN_PARTIAL_FLOATS, 4);
     return 0;
 }
 
@@ -723,7 +724,8 @@ struct Sched {
         a.batch = 8; a.q_bstride = (size_t)128 * 128; a.k_bstride = (size_t)kp * 128; a.vt_bstride = (size_t)128 * kp;
         a.group = 2; a.rows = 2 * ch; a.keys = P + ch; a.scale = 0.08838834764831845f; a.prefix_alloc = P + ch;
         a.out = c->B("decoder_attn"); a.out_tiled = 1; a.out_bcol = 256; a.out_cols32 = 64;
-        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_GQA128_SUFFIX, s), "suffix attn");
+        a.nsplit = c->attn_split > 0 ? c->attn_split : std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
+        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_GQA128_SUFFIX, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024;
         skinny(c->B("decoder_attn"), 2048, ch, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
         SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 2048; g.factor_f32 = 1;
