@@ -1,7 +1,7 @@
-/* rtvla - C ABI of the MI355X (gfx950) Pi0 / Pi05 single-observation forward pass.
+/* rtvla - C ABI of the MI355X (gfx950) Pi0 / Pi05 / DM0 single-observation forward pass.
  *
  * The reference (Dexmal/realtime-vla) has no native layer: its device code is Triton JIT and its
- * "operator interface" is the Python object Pi0Inference / Pi05Inference.  This ABI is what a
+ * "operator interface" is the Python object Pi0Inference / Pi05Inference / DM0Inference.  This ABI is what a
  * Python (ctypes) front end with that object's signature binds instead of the Triton kernels.
  * Every entry point takes plain pointers and sizes, returns an int status (0 = ok, see
  * rtvla_status) and never throws; device memory is always owned by the caller.
@@ -39,16 +39,27 @@ enum rtvla_model { RTVLA_PI0 = 0, RTVLA_PI05 = 1, RTVLA_DM0 = 2 };
 
 /* Static shape set of one inference object.
  * Replaces the constructor arguments and literals of Pi0Inference.__init__
- * (/root/reference/pi0_infer.py:1239-1243, :1289-1290) and Pi05Inference.__init__
- * (/root/reference/pi05_infer.py:531-561, :615-616). */
+ * (/root/reference/pi0_infer.py:1239-1243, :1289-1290), Pi05Inference.__init__
+ * (/root/reference/pi05_infer.py:531-561, :615-616) and DM0Inference.__init__
+ * (/root/reference/dm0_infer.py:965-983).
+ *
+ * RTVLA_DM0 (the reference's third model, dm0_infer.py): num_views images of 728x728 (bf16 NCHW, already normalised),
+ * prompt_len = max_lang_len token ids (int32 "input_ids", looked up in "vision_embed_tokens_w"), a ViT of
+ * vision_layers (23) layers of width 1024 over 2705 tokens per image, two stride-2 convolutions and a projector to
+ * 169 tokens of width 2048 per image, llm_layers (28) causal grouped-query prefix layers and as many action-expert
+ * layers.  Its tensor table is dm0_infer.py:986-1026 by name; the 4-byte tensors among the weights (the folded
+ * LayerNorm biases and column sums, :1013-1018) are fp32, every other weight is bf16.  The caller also binds the three
+ * rotary tables: "vision_rope" bf16 [2705][64] = (cos, sin) per rotation pair of the 2-D embedding (:671-688),
+ * "prefix_rope_weights" [169 views + prompt_len][128] and "decoder_rope_weights" [chunk][128] (:1080-1094). */
 typedef struct rtvla_dims {
     int32_t model;           /* rtvla_model                                                          */
-    int32_t num_views;       /* 1..4 camera views of 224x224x3                                        */
-    int32_t prompt_len;      /* Pi0: rows of language_embeds; Pi05: max_prompt_len (allocated rows)   */
-    int32_t chunk_size;      /* action chunk; Pi0 suffix = chunk+1 rows, Pi05 = chunk rows (<= 64)    */
-    int32_t num_steps;       /* Euler flow steps (the reference hard-codes 10)                        */
-    int32_t vision_layers;   /* SigLIP layers (27)                                                    */
-    int32_t llm_layers;      /* Gemma prefix layers == action-expert layers (18)                      */
+    int32_t num_views;       /* 1..4 camera views of 224x224x3 (DM0: images of 728x728)               */
+    int32_t prompt_len;      /* Pi0: rows of language_embeds; Pi05: max_prompt_len (allocated rows);
+                                DM0: max_lang_len (token ids)                                          */
+    int32_t chunk_size;      /* action chunk; Pi0 suffix = chunk+1 rows, Pi05 / DM0 = chunk rows (<= 64) */
+    int32_t num_steps;       /* Euler flow steps (the reference hard-codes 10; Pi05 / DM0: at most 10) */
+    int32_t vision_layers;   /* SigLIP layers (27); DM0: ViT layers (23)                               */
+    int32_t llm_layers;      /* prefix layers == action-expert layers (18; DM0: 28)                    */
 } rtvla_dims;
 
 /* Stages of the forward schedule, for per-stage execution (layer taps, profiling).
@@ -56,6 +67,8 @@ typedef struct rtvla_dims {
  * PREFIX_LAYER x llm_layers, SUFFIX_INIT, then per step SUFFIX_STEP_BEGIN,
  * SUFFIX_LAYER x llm_layers, SUFFIX_STEP_END. */
 enum rtvla_stage {
+    /* (DM0: dm0_infer.py:695-712 patch embedding + class token + ln_pre; :717-733 one ViT layer; :734-761 the two
+     *  down-sampling convolutions, projector and token embedding; :874-951 one prefix layer; :763-872 the action expert) */
     RTVLA_STAGE_VISION_EMBED = 0,   /* pi0_infer.py:348-364 conv2d_embed_n256_1152_res               */
     RTVLA_STAGE_VISION_LAYER = 1,   /* pi0_infer.py:607-646 one SigLIP layer                         */
     RTVLA_STAGE_PROJECT = 2,        /* pi0_infer.py:753-775 + :1344 final LN, projector, prompt rows */
@@ -68,7 +81,7 @@ enum rtvla_stage {
 
 /* Library version (no reference counterpart): raised whenever a kernel or the schedule changes, so that a
  * measurement recorded for one version is not mistaken for the current kernels. */
-#define RTVLA_VERSION 2
+#define RTVLA_VERSION 3
 int rtvla_version(void);
 
 /* Create a context for one shape set.  Replaces the tensor allocation block of
