@@ -7,7 +7,7 @@
 //                    action-expert suffix pass with its masks (pi0_infer.py:1041-1120, pi05_infer.py:382-478).
 //                    G = 2, HD = 128, 8 K/V heads: DM0's grouped-query attention, causal in the prefix
 //                    (/root/reference/dm0_infer.py:913-918) and unmasked in the action expert (:822-826).
-//                    G = 1, HD = 64, one K/V head per (image, head): DM0's ViT attention (:589-598).
+//                    (DM0's ViT attention, long on both sides, is csrc/flash.hip.)
 //  * vision_kernel - SigLIP attention, 16 heads x 72 per view, 256 keys (pi0_infer.py:588-596).
 //
 // Both compute the transposed logits S^T = K Q^T so that each lane holds 16 keys of ONE query row:
@@ -37,14 +37,19 @@ RTVLA_DEVICE bf16x8 cat44(bf16x4 lo, bf16x4 hi) {
 // where element (row, d) of the output goes: row-major [token][ld_tok] with the G heads of a token side by side (and the
 // batch index split into an outer and an inner part with a stride each), or the fragment-tiled [tokens][32 out_cols32]
 // matrix the action-expert O projection reads
-RTVLA_DEVICE bf16_t* attn_out_ptr(const AttnP& p, int batch, int row, int d, int hd) {
+struct AttnOutRow { bf16_t* base; int tok, col; };
+RTVLA_DEVICE AttnOutRow attn_out_row(const AttnP& p, int batch, int row, int hd) {
     const int tok = row / p.group, sub = row - tok * p.group;
-    if (p.out_tiled) return p.out + ft_index(tok, batch * p.out_bcol + sub * hd + d, p.out_cols32);
+    if (p.out_tiled) return {p.out, tok, batch * p.out_bcol + sub * hd};
     const int bo = batch / p.batch_inner, bi = batch - bo * p.batch_inner;
-    return p.out + (size_t)bo * p.out_ostride + (size_t)bi * p.out_istride + (size_t)tok * p.ld_tok + sub * hd + d;
+    return {p.out + (size_t)bo * p.out_ostride + (size_t)bi * p.out_istride + (size_t)tok * p.ld_tok + sub * hd, tok, 0};
 }
+RTVLA_DEVICE bf16_t* attn_out_at(const AttnP& p, const AttnOutRow& o, int d) {
+    return p.out_tiled ? o.base + ft_index(o.tok, o.col + d, p.out_cols32) : o.base + d;
+}
+RTVLA_DEVICE bf16_t* attn_out_ptr(const AttnP& p, int batch, int row, int d, int hd) { return attn_out_at(p, attn_out_row(p, batch, row, hd), d); }
 
-template <int WAVES, int MQ, int NTK, int HD>
+template <int WAVES, int MQ, int NTK, int HD, bool CAUSAL>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(1, HD == 256 ? 1 : 2)))
 void mqa_kernel(AttnP p) {
     constexpr int KD = HD / 32;                                       // 32-wide steps of the Q K^T contraction
@@ -96,7 +101,7 @@ void mqa_kernel(AttnP p) {
     constexpr int KBS = NTK * 16;                    // keys per block
     int nkb = (p.keys + KBS - 1) / KBS;
     // causal: the last row of this block sees keys up to its own token
-    if (p.causal) nkb = min(nkb, (min(m0 + 16 * MQ, p.rows) - 1) / p.group / KBS + 1);
+    if constexpr (CAUSAL) nkb = min(nkb, (min(m0 + 16 * MQ, p.rows) - 1) / p.group / KBS + 1);
     const int kb_begin = split * p.kb_per_split, kb_end = min(nkb, kb_begin + p.kb_per_split);
     const int keys32 = p.ldvt >> 5;
     bf16x8 kf[NTK][KD];       // K fragments of one key block (A operand of S^T = K Q^T)
@@ -141,6 +146,8 @@ void mqa_kernel(AttnP p) {
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq) {
             const int row = m0 + mq * 16 + r;
+            int own = 0;                                      // causal: the row's own token, the last key it sees
+            if constexpr (CAUSAL) own = row / p.group;
             float mx = NEG_BIG;
             bool vis[NTK][4];
 #pragma unroll
@@ -151,7 +158,7 @@ void mqa_kernel(AttnP p) {
                     bool ok = key < p.keys;
                     if (key < p.prefix_alloc) ok = ok && key < vl;
                     else ok = ok && (row >= p.state_rows || key == p.prefix_alloc);
-                    if (p.causal) ok = ok && key <= row / p.group;
+                    if constexpr (CAUSAL) ok = ok && key <= own;
                     vis[nt][v] = ok;
                     const float s = ok ? st[mq][nt][v] * p.scale : NEG_BIG;
                     st[mq][nt][v] = s;
@@ -224,6 +231,7 @@ void mqa_kernel(AttnP p) {
         for (int ww = 0; ww < WAVES; ++ww) lt += ls[(ww * MQ + mq) * 16 + r];
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         const int row = m0 + mq * 16 + r;
+        const AttnOutRow orow = attn_out_row(p, batch, min(row, p.rows - 1), HD);
         if (nsplit > 1 && w == 0 && g == 0) { mine[mq * REC + DT * 256 + r] = mgl[mq]; mine[mq * REC + DT * 256 + 16 + r] = lt; }
         for (int dt = w; dt < DT; dt += WAVES) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
@@ -232,7 +240,7 @@ void mqa_kernel(AttnP p) {
             if (nsplit > 1) {
                 *(f32x4*)(mine + mq * REC + (dt * 64 + lane) * 4) = t;
             } else if (row < p.rows) {
-                store4(attn_out_ptr(p, batch, row, dt * 16 + 4 * g, HD), pack4(t * inv));
+                store4(attn_out_at(p, orow, dt * 16 + 4 * g), pack4(t * inv));
             }
         }
     }
@@ -362,10 +370,11 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     }
 }
 
-template <int WAVES, int MQ, int NTK, int HD>
+template <int WAVES, int MQ, int NTK, int HD, bool CAUSAL = false>
 int launch_mqa_inst(AttnP p, hipStream_t s) {
     const size_t smem = (size_t)WAVES * (HD / 16) * 64 * 16 + (size_t)2 * WAVES * MQ * 16 * 4;
-    auto kern = mqa_kernel<WAVES, MQ, NTK, HD>;
+    auto kern = mqa_kernel<WAVES, MQ, NTK, HD, CAUSAL>;
+    if (CAUSAL != (p.causal != 0)) return 1;
     if (smem > 65536) {
         static bool done = false;
         if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
@@ -398,9 +407,8 @@ int launch_mqa_attention(const AttnP& p0, int variant, hipStream_t s) {
     switch (variant) {                                          // template: waves, row tiles per workgroup, 16-key tiles per wave round, head width
         case ATTN_PREFIX: return launch_mqa_inst<4, 2, 2, 256>(p, s);
         case ATTN_SUFFIX: return launch_mqa_inst<4, 1, 2, 256>(p, s);
-        case ATTN_GQA128_PREFIX: return launch_mqa_inst<4, 2, 2, 128>(p, s);
+        case ATTN_GQA128_PREFIX: return launch_mqa_inst<4, 2, 2, 128, true>(p, s);
         case ATTN_GQA128_SUFFIX: return launch_mqa_inst<4, 1, 2, 128>(p, s);
-        case ATTN_VIT64: return launch_mqa_inst<4, 4, 2, 64>(p, s);
     }
     return 2;
 }

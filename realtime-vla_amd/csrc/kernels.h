@@ -144,8 +144,8 @@ struct AttnP {
     RTVLA_KO_FIELD
 };
 // Gemma (HD 256): many rows, two row tiles per workgroup / few rows, one row tile and a key split; DM0 grouped-query (HD 128)
-// prefix and suffix; DM0 ViT (HD 64)
-enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1, ATTN_GQA128_PREFIX, ATTN_GQA128_SUFFIX, ATTN_VIT64 };
+// prefix and suffix (the ViT attention, HD 64, is launch_flash_attention)
+enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1, ATTN_GQA128_PREFIX, ATTN_GQA128_SUFFIX };
 int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s);
 // long sequences on both sides (csrc/flash.hip): 128 query rows per workgroup, K / V^T tiles shared through LDS; hd = 64
 int launch_flash_attention(const AttnP& p, int hd, hipStream_t s);
