@@ -29,7 +29,7 @@ __global__ void dm0_im2col_nchw_kernel(const bf16_t* __restrict__ img, bf16_t* _
 // ln_pre in place: (x - mean) * rsqrt(E[x^2] - mean^2 + 1e-5) * w + b  (dm0_infer.py:699-712, :442-454, :561-579).
 __global__ __launch_bounds__(256)
 void dm0_embed_ln_kernel(const bf16_t* __restrict__ conv, const bf16_t* __restrict__ cls, const bf16_t* __restrict__ pos,
-                         const bf16_t* __restrict__ w, const bf16_t* __restrict__ b, bf16_t* __restrict__ x) {
+                         const bf16_t* __restrict__ w, const bf16_t* __restrict__ b, bf16_t* __restrict__ x, int x_img_rows) {
     __shared__ float red[2][4];
     const int row = blockIdx.x, tid = threadIdx.x;
     const int n = row / DM0_SEQ, tok = row - n * DM0_SEQ;
@@ -45,7 +45,7 @@ void dm0_embed_ln_kernel(const bf16_t* __restrict__ conv, const bf16_t* __restri
     const float var = (red[1][0] + red[1][1] + red[1][2] + red[1][3]) * (1.0f / 1024.0f) - mean * mean;
     const float rstd = rsqrtf(var + 1e-5f);
     const bf16x4 ww = load4(w + tid * 4), bb = load4(b + tid * 4);
-    store4(x + (size_t)row * 1024 + tid * 4, pack4((v[0] - mean) * rstd * bf2f(ww[0]) + bf2f(bb[0]), (v[1] - mean) * rstd * bf2f(ww[1]) + bf2f(bb[1]),
+    store4(x + ((size_t)n * x_img_rows + tok) * 1024 + tid * 4, pack4((v[0] - mean) * rstd * bf2f(ww[0]) + bf2f(bb[0]), (v[1] - mean) * rstd * bf2f(ww[1]) + bf2f(bb[1]),
                                                    (v[2] - mean) * rstd * bf2f(ww[2]) + bf2f(bb[2]), (v[3] - mean) * rstd * bf2f(ww[3]) + bf2f(bb[3])));
 }
 
@@ -135,8 +135,8 @@ void launch_dm0_im2col_nchw(const bf16_t* images, bf16_t* patches, int ldp, int 
     hipLaunchKernelGGL(dm0_im2col_nchw_kernel, dim3((total + 255) / 256), dim3(256), 0, s, images, patches, ldp, rows);
 }
 
-void launch_dm0_embed_ln(const bf16_t* conv, const bf16_t* cls, const bf16_t* pos, const bf16_t* w, const bf16_t* b, bf16_t* x, int n_images, hipStream_t s) {
-    hipLaunchKernelGGL(dm0_embed_ln_kernel, dim3(n_images * DM0_SEQ), dim3(256), 0, s, conv, cls, pos, w, b, x);
+void launch_dm0_embed_ln(const bf16_t* conv, const bf16_t* cls, const bf16_t* pos, const bf16_t* w, const bf16_t* b, bf16_t* x, int x_img_rows, int n_images, hipStream_t s) {
+    hipLaunchKernelGGL(dm0_embed_ln_kernel, dim3(n_images * DM0_SEQ), dim3(256), 0, s, conv, cls, pos, w, b, x, x_img_rows);
 }
 
 void launch_dm0_im2col3x3(const bf16_t* in, int img_rows, int row0, int in_h, int in_w, int C, bf16_t* col, int n_images, hipStream_t s) {

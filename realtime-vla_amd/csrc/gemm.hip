@@ -291,6 +291,7 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
         if (m >= p.M) continue;
 #pragma unroll
         for (int j = 0; j < HALF; ++j) {
+          uint2 qk[4];                                                  // (EPI_VIT_QKV_ROPE: the rotated values of the four groups)
 #pragma unroll
           for (int grp = 0; grp < 4; ++grp) {
             const int n0 = tile_of[j] * 32 + 8 * grp + 4 * h;
@@ -336,23 +337,52 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
                 }
             } else if constexpr (EPI == EPI_VIT_QKV_ROPE) {
                 // DM0 ViT (dm0_infer.py:589-598): + fp32 bias, rounded to bf16 as the reference's QKV buffer is, then the 2-D rotary
-                // embedding on Q and K; per (image, head) Q and K as fragment-tiled [seq_pad][64], V^T as [64][seq_pad]
+                // embedding on Q and K; per (image, head) Q and K as fragment-tiled [seq_pad][64], V^T as [64][seq_pad].  The rows
+                // are laid out as seq_pad (a multiple of 32) per image, so a 32-row tile is one 32-key block of one image.
                 v += *(const f32x4*)(p.bias_f32 + n0);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = round_bf16(v[e]);
                 const int which = n0 >> 10, cc = n0 & 1023, head = cc >> 6, d = cc & 63;
-                const int img = m / p.seq, tok = m - img * p.seq;
+                const int img = m / p.seq_pad, tok = m - img * p.seq_pad;
                 const size_t vh = (size_t)(img * 16 + head);
                 if (which < 2) {
-                    const bf16x4 cs = load4(p.rope + (size_t)tok * 64 + d);
+                    const bf16x4 cs = load4(p.rope + (size_t)min(tok, p.seq - 1) * 64 + d);
                     const float c0 = bf2f(cs[0]), s0 = bf2f(cs[1]), c1 = bf2f(cs[2]), s1 = bf2f(cs[3]);
                     const f32x4 w = v;
                     v[0] = w[0] * c0 - w[1] * s0; v[1] = w[1] * c0 + w[0] * s0;
                     v[2] = w[2] * c1 - w[3] * s1; v[3] = w[3] * c1 + w[2] * s1;
-                    store4((which == 0 ? p.q : p.k) + vh * ((size_t)p.seq_pad * 64) + ft_index(tok, d, 2), pack4(v));
-                } else {
+                    // lanes h = 0 / 1 of a row hold the two halves of every 8-wide chunk: swap halves so that each lane owns two
+                    // whole 16-byte pieces of the fragment-tiled Q / K
+                    const bf16x4 pk = pack4(v);
+                    qk[grp] = *(const uint2*)&pk;
+                    if (grp == 3) {
+                        bf16_t* const dst = (which == 0 ? p.q : p.k) + vh * ((size_t)p.seq_pad * 64);
+                        const int d0 = (tile_of[j] * 32) & 63;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) p.vt[vh * ((size_t)64 * p.seq_pad) + vt_index(d + e, tok, p.seq_pad >> 5)] = f2bf(v[e]);
+                        for (int pr = 0; pr < 2; ++pr) {
+                            const uint2 keep = h ? qk[2 * pr + 1] : qk[2 * pr], send = h ? qk[2 * pr] : qk[2 * pr + 1];
+                            const uint2 recv = {(unsigned)__shfl_xor((int)send.x, 32, 64), (unsigned)__shfl_xor((int)send.y, 32, 64)};
+                            *(uint4*)(dst + ft_index(tok, d0 + 8 * (2 * pr + h), 2)) = h ? uint4{recv.x, recv.y, keep.x, keep.y} : uint4{keep.x, keep.y, recv.x, recv.y};
+                        }
+                    }
+                } else {
+                    // V^T: the wave's 32 keys x 32 d tile is transposed through a private 2.3 KB of LDS ([d][key], 72-byte pitch)
+                    // so that it leaves as whole 16-byte pieces of the permuted-key fragments instead of 2-byte stores
+                    volatile bf16_t* tb = (volatile bf16_t*)(smem_raw + wn * 2304);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) tb[(8 * grp + 4 * h + e) * 36 + r] = f2bf(v[e]);
+                    if (grp == 3) {
+                        const int tok0 = tok - r;                                   // first key of the tile: a multiple of 32
+                        const int d0 = (tile_of[j] * 32) & 63;                      // head-local d of the tile's first column
+                        const int gq = lane >> 4, rq = lane & 15;
+#pragma unroll
+                        for (int dt = 0; dt < 2; ++dt) {
+                            const volatile uint2* src = (const volatile uint2*)(smem_raw + wn * 2304 + (16 * dt + rq) * 72 + gq * 8);
+                            const uint2 lo = {src[0].x, src[0].y}, hi = {src[4].x, src[4].y};       // keys 4 gq .. +3 and 16 + 4 gq .. +3
+                            const size_t frag = (size_t)(((d0 >> 4) + dt) * (p.seq_pad >> 5) + (tok0 >> 5)) * 64 + lane;
+                            *(uint4*)(p.vt + vh * ((size_t)64 * p.seq_pad) + frag * 8) = uint4{lo.x, lo.y, hi.x, hi.y};
+                        }
+                    }
                 }
             } else if constexpr (EPI == EPI_VIS_QKV) {
                 const bf16x4 b = load4(p.bias + n0);

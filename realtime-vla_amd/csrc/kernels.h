@@ -162,7 +162,7 @@ void launch_fill_bf16(bf16_t* p, size_t n, float v, hipStream_t s);
 
 // ----- DM0 (csrc/dm0.hip) ---------------------------------------------------------------------
 void launch_dm0_im2col_nchw(const bf16_t* images, bf16_t* patches, int ldp, int n_images, hipStream_t s);
-void launch_dm0_embed_ln(const bf16_t* conv, const bf16_t* cls, const bf16_t* pos, const bf16_t* w, const bf16_t* b, bf16_t* x, int n_images, hipStream_t s);
+void launch_dm0_embed_ln(const bf16_t* conv, const bf16_t* cls, const bf16_t* pos, const bf16_t* w, const bf16_t* b, bf16_t* x, int x_img_rows, int n_images, hipStream_t s);
 void launch_dm0_im2col3x3(const bf16_t* in, int img_rows, int row0, int in_h, int in_w, int C, bf16_t* col, int n_images, hipStream_t s);
 void launch_dm0_gather_rows(const bf16_t* table, int table_rows, const int* ids, bf16_t* dst, int rows, hipStream_t s);
 void launch_dm0_qknorm_rope(const bf16_t* qkv, int ld, const float* factor, const bf16_t* x_tiled, const bf16_t* qw, const bf16_t* kw, const bf16_t* rope,

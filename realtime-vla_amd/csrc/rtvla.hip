@@ -314,7 +314,7 @@ int build_tables(rtvla_ctx* c) {
 
 // DM0 (/root/reference/dm0_infer.py:965-1076): tensors under the reference's names, then the workspace.
 constexpr int DM0_SEQ = 2705;          // 52 x 52 patches + class token per image
-constexpr int DM0_SEQ_PAD = 2720;      // padded to the 32-key blocks of the attention kernel
+constexpr int DM0_SEQ_PAD = 2720;      // rows per image in every ViT buffer: whole 32-row GEMM tiles and 32-key attention blocks
 constexpr int DM0_TOK = 169;           // tokens per image after the two stride-2 convolutions
 
 int build_tables_dm0(rtvla_ctx* c) {
@@ -390,7 +390,7 @@ int build_tables_dm0(rtvla_ctx* c) {
     c->add_tiled("t_decoder_action_mlp_w", 1024, 1024, 1);
     c->add_tiled("t_decoder_out_proj_w", 1024, 32, 1);
     c->act_begin = c->ws_bytes;
-    const int64_t M = n * DM0_SEQ;
+    const int64_t M = n * DM0_SEQ_PAD;                                       // every image owns 2720 rows of the row-major ViT buffers
     c->add_buf("const_ones", 1, 1024, 1024);
     c->add_buf("const_zeros", 1, 6144, 6144);
     c->add_buf("vision_patches", n * 2704, PATCH_LD, PATCH_LD);
@@ -615,13 +615,13 @@ struct Sched {
 
     // dm0_infer.py:695-712: patch embedding, class token, position embedding, ln_pre; then the first layer's LayerNorm
     void dm0_vision_embed() {
-        const int n = d.num_views, M = n * DM0_SEQ;
+        const int n = d.num_views, M = n * DM0_SEQ_PAD;
         if (c->want("im2col")) { launch_dm0_im2col_nchw(c->W("images"), c->B("vision_patches"), PATCH_LD, n, s); c->note(0, "im2col"); }
         GemmP e{}; e.out = c->B("vision_conv1_buf"); e.ldo = 1024; e.bias = c->B("const_zeros");
         gemm(c->B("vision_patches"), PATCH_LD, n * 2704, n * 2704, c->TW("t_vision_conv1_w_t"), nullptr, 588, 1024, EPI_BIAS, e, "patch embed");
         if (c->want("class + pos + ln_pre")) {
             launch_dm0_embed_ln(c->B("vision_conv1_buf"), c->W("vision_class_embedding"), c->W("vision_pos_emb"), c->W("vision_ln_pre_w"), c->W("vision_ln_pre_b"),
-                                c->B("vision_x_2d"), n, s);
+                                c->B("vision_x_2d"), DM0_SEQ_PAD, n, s);
             c->note(0, "class + pos + ln_pre");
         }
         reduce(M, 1024, nullptr, c->B("vision_x_2d"), 1024, nullptr, 0, c->B("vision_x_norm"), 1024, NORM_LAYER, c->B("const_ones"), c->B("const_zeros"), 1e-5f, 0, "vit LN0");
@@ -630,7 +630,7 @@ struct Sched {
     // dm0_infer.py:718-736.  The LayerNorm scale and shift are folded into the weights; the rows are normalised by the reduce
     // kernel (x_norm), which equals the reference's  rstd (x W' - mean colsum(W')) + b'  up to the rounding of x_norm.
     void dm0_vision_layer(int i) {
-        const int n = d.num_views, M = n * DM0_SEQ;
+        const int n = d.num_views, M = n * DM0_SEQ_PAD;
         GemmP e{}; e.bias_f32 = WF("vision_fused_qkv_b", 3072, i); e.rope = c->W("vision_rope"); e.seq = DM0_SEQ; e.seq_pad = DM0_SEQ_PAD;
         e.q = c->B("vision_Q"); e.k = c->B("vision_K"); e.vt = c->B("vision_Vt");
         gemm(c->B("vision_x_norm"), 1024, M, M, c->TW("t_vision_fused_qkv_w", i), nullptr, 1024, 3072, EPI_VIT_QKV_ROPE, e, "vit qkv");
@@ -638,7 +638,7 @@ struct Sched {
         a.q = c->B("vision_Q"); a.k = c->B("vision_K"); a.vt = c->B("vision_Vt"); a.ldvt = DM0_SEQ_PAD;
         a.batch = n * 16; a.q_bstride = a.k_bstride = (size_t)DM0_SEQ_PAD * 64; a.vt_bstride = (size_t)64 * DM0_SEQ_PAD;
         a.group = 1; a.rows = DM0_SEQ; a.keys = DM0_SEQ; a.scale = 0.125f; a.prefix_alloc = DM0_SEQ;
-        a.out = c->B("vision_attn"); a.ld_tok = 1024; a.batch_inner = 16; a.out_ostride = (size_t)DM0_SEQ * 1024; a.out_istride = 64;
+        a.out = c->B("vision_attn"); a.ld_tok = 1024; a.batch_inner = 16; a.out_ostride = (size_t)DM0_SEQ_PAD * 1024; a.out_istride = 64;
         if (c->want("vit attn")) c->note(launch_flash_attention(a, 64, s), "vit attn");
         gemm(c->B("vision_attn"), 1024, M, M, c->TW("t_vision_out_proj_w", i), nullptr, 1024, 1024, EPI_PARTIAL, GemmP{}, "vit o");
         reduce(M, 1024, c->W("vision_out_proj_b", 1024, i), c->B("vision_x_2d"), 1024, c->B("vision_x_2d"), 1024, c->B("vision_x_norm"), 1024,
@@ -654,7 +654,7 @@ struct Sched {
     // factor of the first prefix layer
     void dm0_project() {
         const int n = d.num_views, P = c->S_e, T = n * DM0_TOK;
-        if (c->want("im2col ds1")) { launch_dm0_im2col3x3(c->B("vision_x_2d"), DM0_SEQ, 1, 52, 52, 1024, c->B("vision_col1"), n, s); c->note(0, "im2col ds1"); }
+        if (c->want("im2col ds1")) { launch_dm0_im2col3x3(c->B("vision_x_2d"), DM0_SEQ_PAD, 1, 52, 52, 1024, c->B("vision_col1"), n, s); c->note(0, "im2col ds1"); }
         GemmP e{}; e.out = c->B("vision_mm1"); e.ldo = 2048; e.bias = c->W("vision_ds1_b");
         gemm(c->B("vision_col1"), 9216, n * 676, n * 676, c->TW("t_vision_ds1_w"), nullptr, 9216, 2048, EPI_BIAS, e, "ds1");
         if (c->want("im2col ds2")) { launch_dm0_im2col3x3(c->B("vision_mm1"), 676, 0, 26, 26, 2048, c->B("vision_col2"), n, s); c->note(0, "im2col ds2"); }

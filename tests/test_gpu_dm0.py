@@ -45,6 +45,15 @@ class Case:
         self.e.run_stage(stage, layer, step)
         torch.cuda.synchronize()
 
+    def vit(self, name):
+        """The valid rows of a row-major ViT buffer (every image owns 2720 rows, 2705 of them tokens)."""
+        b = self.B[name]
+        return b.view(self.n, 2720, b.shape[1])[:, :2705].reshape(self.n * 2705, b.shape[1])
+
+    def set_vit(self, name, x):
+        b = self.B[name]
+        b.view(self.n, 2720, b.shape[1])[:, :2705].copy_(bf(x).view(self.n, 2705, b.shape[1]))
+
     def dec_x(self):
         from _engine import untile_ft
         return untile_ft(self.B["decoder_x"], 64, 1024)[:50]
@@ -85,10 +94,10 @@ class Case:
                 b = t32[tap][:rows] if rows is not None else t32[tap]
                 odrift[name] = rel(a, b)
         self.run(c.STAGE_VISION_EMBED)
-        note("vision_embed", self.B["vision_x_2d"], "vision_embed")
+        note("vision_embed", self.vit("vision_x_2d"), "vision_embed")
         for i in range(self.VL):
             self.run(c.STAGE_VISION_LAYER, i)
-            note("vision_x/%d" % i, self.B["vision_x_2d"], "vision_x/%d" % i)
+            note("vision_x/%d" % i, self.vit("vision_x_2d"), "vision_x/%d" % i)
         self.run(c.STAGE_PROJECT)
         note("prefix_x0", self.B["prefix_x"], "prefix_x0")
         for i in range(self.LL):
@@ -111,14 +120,14 @@ class Case:
         errs = {}
         self.stage_inputs()
         self.run(c.STAGE_VISION_EMBED)
-        errs["vision_embed"] = rel(self.B["vision_x_2d"], t["vision_embed"])
+        errs["vision_embed"] = rel(self.vit("vision_x_2d"), t["vision_embed"])
         for i in range(self.VL):
             x = t["vision_embed"] if i == 0 else t["vision_x/%d" % (i - 1)]
             mean, rstd = o.ln_stats(x)
-            self.B["vision_x_2d"].copy_(bf(x)); self.B["vision_x_norm"].copy_(bf((x - mean) * rstd))
+            self.set_vit("vision_x_2d", x); self.set_vit("vision_x_norm", (x - mean) * rstd)
             self.run(c.STAGE_VISION_LAYER, i)
-            errs["vision_layer/%d" % i] = rel(self.B["vision_x_2d"], t["vision_x/%d" % i])
-        self.B["vision_x_2d"].copy_(bf(t["vision_x/%d" % (self.VL - 1)]))
+            errs["vision_layer/%d" % i] = rel(self.vit("vision_x_2d"), t["vision_x/%d" % i])
+        self.set_vit("vision_x_2d", t["vision_x/%d" % (self.VL - 1)])
         self.run(c.STAGE_PROJECT)
         errs["project"] = rel(self.B["prefix_x"], t["prefix_x0"])
         for i in range(self.LL):
