@@ -10,7 +10,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librtvla.so")
 SOURCES = ["gemm.hip", "skinny.hip", "attention.hip", "misc.hip", "dm0.hip", "flash.hip", "rtvla.hip", "transforms.hip"]
 # bit-exact parity with host arithmetic (Pillow, numpy): no fused multiply-adds in these files
-EXTRA = {"transforms.hip": ["-ffp-contract=off"]}
+# flash.hip: MFMA results in ordinary VGPRs (the softmax reads every logit; the accumulator-register form costs a copy each)
+EXTRA = {"transforms.hip": ["-ffp-contract=off"], "flash.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-unused-value",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
