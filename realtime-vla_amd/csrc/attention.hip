@@ -80,6 +80,8 @@ void mqa_kernel(AttnP p) {
 
     int vl = p.prefix_alloc;
     if (p.valid_len) vl = max(0, min(*p.valid_len, p.prefix_alloc));
+    const int vis_lim = min(vl, p.keys);                             // keys below this are visible to every row (causal aside)
+    const float sc2 = p.scale * 1.4426950408889634f;
 
     bf16x8 qf[MQ][KD];
 #pragma unroll
@@ -143,46 +145,60 @@ void mqa_kernel(AttnP p) {
         load_k(kb_next);                                     // next block's K flies during softmax and P V
         __builtin_amdgcn_sched_barrier(0);
         bf16x8 pb[MQ][NTK / 2];
+        bool full = key0 + KBS <= vis_lim;
+        if constexpr (CAUSAL) full = full && key0 + KBS - 1 <= m0 / p.group;
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq) {
             const int row = m0 + mq * 16 + r;
             int own = 0;                                      // causal: the row's own token, the last key it sees
             if constexpr (CAUSAL) own = row / p.group;
+            // logits in the base-2 domain (scale * log2 e folded into one multiply); a block every row sees whole (all but the
+            // last of a prefix pass) takes the path without mask arithmetic
             float mx = NEG_BIG;
             bool vis[NTK][4];
+            if (full) {
 #pragma unroll
-            for (int nt = 0; nt < NTK; ++nt)
+                for (int nt = 0; nt < NTK; ++nt)
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int key = key0 + nt * 16 + 4 * g + v;
-                    bool ok = key < p.keys;
-                    if (key < p.prefix_alloc) ok = ok && key < vl;
-                    else ok = ok && (row >= p.state_rows || key == p.prefix_alloc);
-                    if constexpr (CAUSAL) ok = ok && key <= own;
-                    vis[nt][v] = ok;
-                    const float s = ok ? st[mq][nt][v] * p.scale : NEG_BIG;
-                    st[mq][nt][v] = s;
-                    mx = fmaxf(mx, s);
-                }
+                    for (int v = 0; v < 4; ++v) { st[mq][nt][v] *= sc2; mx = fmaxf(mx, st[mq][nt][v]); vis[nt][v] = true; }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NTK; ++nt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int key = key0 + nt * 16 + 4 * g + v;
+                        bool ok = key < p.keys;
+                        if (key < p.prefix_alloc) ok = ok && key < vl;
+                        else ok = ok && (row >= p.state_rows || key == p.prefix_alloc);
+                        if constexpr (CAUSAL) ok = ok && key <= own;
+                        vis[nt][v] = ok;
+                        const float s = ok ? st[mq][nt][v] * sc2 : NEG_BIG;
+                        st[mq][nt][v] = s;
+                        mx = fmaxf(mx, s);
+                    }
+            }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float mnew = fmaxf(mrun[mq], mx);
-            const float alpha = __expf(mrun[mq] - mnew);
+            if (__any(mx > mrun[mq])) {                       // the accumulator is rescaled only when some row's maximum grew
+                const float mnew = fmaxf(mrun[mq], mx);
+                const float alpha = __builtin_amdgcn_exp2f(mrun[mq] - mnew);
+                lrun[mq] *= alpha;
+                mrun[mq] = mnew;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[mq][dt] *= alpha;
+            }
             float sum = 0.f;
 #pragma unroll
             for (int nt = 0; nt < NTK; ++nt)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const float e = vis[nt][v] ? __expf(st[mq][nt][v] - mnew) : 0.f;
+                    const float e = vis[nt][v] ? __builtin_amdgcn_exp2f(st[mq][nt][v] - mrun[mq]) : 0.f;
                     st[mq][nt][v] = e;
                     sum += e;
                 }
             sum += __shfl_xor(sum, 16, 64);
             sum += __shfl_xor(sum, 32, 64);
-            lrun[mq] = lrun[mq] * alpha + sum;
-            mrun[mq] = mnew;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o[mq][dt] *= alpha;
+            lrun[mq] += sum;
 #pragma unroll
             for (int kk = 0; kk < NTK / 2; ++kk) pb[mq][kk] = cat44(pack4(st[mq][2 * kk]), pack4(st[mq][2 * kk + 1]));
         }
@@ -210,7 +226,7 @@ void mqa_kernel(AttnP p) {
         float mg = NEG_BIG;
 #pragma unroll
         for (int ww = 0; ww < WAVES; ++ww) mg = fmaxf(mg, ms[(ww * MQ + mq) * 16 + r]);
-        const float sc = __expf(mrun[mq] - mg);
+        const float sc = __builtin_amdgcn_exp2f(mrun[mq] - mg);
         lrun[mq] *= sc;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[mq][dt] *= sc;
@@ -275,7 +291,7 @@ void attn_merge_kernel(AttnP p, int nsplit) {
         f32x4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int sp = 0; sp < NS; ++sp) {
-            const float wgt = sp < nsplit ? __expf(ms[sp] - mg) : 0.f;
+            const float wgt = sp < nsplit ? __builtin_amdgcn_exp2f(ms[sp] - mg) : 0.f;      // the maxima are base-2 logits
             lt += wgt * ls[sp];
             t += os[sp] * wgt;
         }
@@ -300,7 +316,7 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     const int quarter = blk & 3, vh = blk >> 2, head = vh & 15, view = vh >> 4;
     const int mtile = quarter * 4 + w;                             // 16-row tile of this wave inside the view
     const int row = view * 256 + mtile * 16 + r;                   // query token (global row)
-    const float scale = 0.11785113019775792f;                      // 1 / sqrt(72)
+    const float scale = 0.11785113019775792f * 1.4426950408889634f; // 1 / sqrt(72), in the base-2 domain
 
     const bf16_t* qb = q + (size_t)vh * (256 * 96) + lane * 8;
     const bf16_t* kb_ = k + (size_t)vh * (256 * 96) + lane * 8;
@@ -341,23 +357,27 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
             for (int v = 0; v < 4; ++v) { st[nt][v] *= scale; mx = fmaxf(mx, st[nt][v]); }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float mnew = fmaxf(mrun, mx);
-        const float alpha = __expf(mrun - mnew);
+        if (__any(mx > mrun)) {
+            const float mnew = fmaxf(mrun, mx);
+            const float alpha = __builtin_amdgcn_exp2f(mrun - mnew);
+            lrun *= alpha;
+            mrun = mnew;
+#pragma unroll
+            for (int dt = 0; dt < 5; ++dt) o[dt] *= alpha;
+        }
         float sum = 0.f;
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) { st[nt][v] = __expf(st[nt][v] - mnew); sum += st[nt][v]; }
+            for (int v = 0; v < 4; ++v) { st[nt][v] = __builtin_amdgcn_exp2f(st[nt][v] - mrun); sum += st[nt][v]; }
         sum += __shfl_xor(sum, 16, 64);
         sum += __shfl_xor(sum, 32, 64);
-        lrun = lrun * alpha + sum;
-        mrun = mnew;
+        lrun += sum;
         bf16x8 pb[2];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) pb[kk] = cat44(pack4(st[2 * kk]), pack4(st[2 * kk + 1]));
 #pragma unroll
         for (int dt = 0; dt < 5; ++dt) {
-            o[dt] *= alpha;
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) o[dt] = mfma16(vf[dt][kb * 2 + kk], pb[kk], o[dt]);
         }
