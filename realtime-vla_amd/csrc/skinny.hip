@@ -102,7 +102,10 @@ void skinny_kernel(SkinnyP p) {
 #pragma unroll
                 for (int i = 0; i < SK_CH; ++i)
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) { const float x = bf2f(a[0][mt][i][j]); s += x * x; }
+                    for (int j = 0; j < 8; j += 2) {                       // v_dot2_f32_bf16: two squares per instruction, no conversions
+                        const bf16x2 x2 = {a[0][mt][i][j], a[0][mt][i][j + 1]};
+                        s = __builtin_amdgcn_fdot2_f32_bf16(x2, x2, s, false);
+                    }
                 s += __shfl_xor(s, 16, 64);
                 s += __shfl_xor(s, 32, 64);
                 ss[mt] = s;
