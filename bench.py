@@ -155,7 +155,7 @@ def bench_dm0(args, dev, desc, views, lang, chunk):
     roofline = None
     if fc:
         tf = fc_flop / (fc[1] * 1e-6) / 1e12
-        roofline = {"bound": "mfma", "kernel": "ViT MLP up-projection with folded LayerNorm and GELU (gemm_mfma_kernel), M=%d K=1024 N=4096" % M,
+        roofline = {"bound": "mfma", "kernel": "ViT MLP up-projection with folded LayerNorm and GELU (gemm8_kernel), M=%d K=1024 N=4096" % M,
                     "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS, 4),
                     "launch_ms": round(fc[1] / 1e3, 4), "traffic": None, "kernel_variant": fc[0],
                     "algorithmic_bytes": 2.0 * (M * 1024 + 1024 * 4096 + M * 4096)}

@@ -8,7 +8,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librtvla.so")
-SOURCES = ["gemm.hip", "skinny.hip", "attention.hip", "misc.hip", "dm0.hip", "flash.hip", "rtvla.hip", "transforms.hip"]
+SOURCES = ["gemm.hip", "gemm8.hip", "skinny.hip", "attention.hip", "misc.hip", "dm0.hip", "flash.hip", "rtvla.hip", "transforms.hip"]
 # bit-exact parity with host arithmetic (Pillow, numpy): no fused multiply-adds in these files
 # flash.hip: MFMA results in ordinary VGPRs (the softmax reads every logit; the accumulator-register form costs a copy each)
 EXTRA = {"transforms.hip": ["-ffp-contract=off"], "flash.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}

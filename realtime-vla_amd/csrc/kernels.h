@@ -69,10 +69,13 @@ struct GemmP {
 // workgroup tile (rows x columns), 4 waves each owning 64 columns (two 32-column MFMA tiles).  The tiles of 128 rows and
 // more by 256 columns are upper bounds: their launches mix row blocks of that many and of 32 fewer rows so that the
 // blocks cover ceil(M / 32) 32-row tiles exactly.
-enum GemmTile { TILE_224x256 = 0, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_64x128, TILE_128x128, TILE_COUNT };
+enum GemmTile { TILE_224x256 = 0, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_64x128, TILE_128x128,
+                // the same 256-column tiles computed by eight waves (csrc/gemm8.hip), row-major epilogues only
+                TILE8_256x256, TILE8_224x256, TILE8_192x256, TILE8_128x256, TILE_COUNT };
 int gemm_tile_bm(int tile);
 int gemm_tile_bn(int tile);
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s);
+int launch_gemm8(const GemmP& p, int epi, int tile, hipStream_t s);
 
 // ----- split-K reduce + bias + residual (+ gate) + normalisation -----------------------
 enum NormMode { NORM_NONE = 0, NORM_RMS, NORM_LAYER };

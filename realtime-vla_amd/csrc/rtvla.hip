@@ -121,7 +121,7 @@ constexpr int64_t ATTN_PARTIAL_FLOATS = 32 * 16 * (16 * 64 * 4 + 32);   // 32 ro
 // workgroup); tiles of 64 rows run two workgroups per CU, which then share the MFMA pipe but overlap
 // their load latency; all workgroups together cannot pull more than ~20 TB/s out of L2; every launch pays a
 // fixed ramp and an epilogue that grows with the tile; split-K adds the reduce pass over the fp32 partials.
-TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what) {
+TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what, bool plain = false) {
     static const int tiles[] = {TILE_224x256, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};
     static const int splits[] = {1, 2, 3, 4, 6, 8};
 #ifdef RTVLA_TUNING
@@ -133,6 +133,9 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
         return c;
     }
 #endif
+    // measured (M = 8115, K = 1024, N = 4096, bias + GELU): the eight-wave 256 x 256 tile takes 84-89 us where the best four-wave
+    // tile takes 98-101 us; with 788 rows, with the gated epilogues and with fp32 split-K partials the four-wave tiles win
+    if (plain && M >= 4096 && stages <= 32 && ncols16 >= 128) return TileChoice{TILE8_256x256, 1};      // plain: bias (+ GELU) epilogue
     double best = 1e30; TileChoice bc{TILE_128x256, 1};
     for (int tile : tiles) {
         const int bm = gemm_tile_bm(tile);
@@ -441,7 +444,7 @@ struct Sched {
         GemmP p = extra;
         p.A = A; p.lda = lda; p.a_rows = a_rows; p.M = M; p.B0 = B0; p.B1 = B1;
         p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.bgroup = bgroup;
-        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU || epi == EPI_SWIGLU, epi == EPI_PARTIAL, what);
+        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU || epi == EPI_SWIGLU, epi == EPI_PARTIAL, what, epi == EPI_BIAS || epi == EPI_BIAS_GELU);
         p.nsplit = tc.nsplit;
         if (epi == EPI_PARTIAL) {
             p.partial = c->B<float>("splitk_partial"); p.ldp = N; p.pstride = (size_t)M * N;
@@ -450,7 +453,7 @@ struct Sched {
         if (c->want(what)) {
             // the name a measurement reports carries the kernel variant: block tile and split-K factor
             c->last_name = std::string(what) + " [" + std::to_string(gemm_tile_bm(tc.tile)) + "x" + std::to_string(gemm_tile_bn(tc.tile)) +
-                           " split " + std::to_string(tc.nsplit) + "]";
+                           (tc.tile >= TILE8_256x256 ? " 8 waves" : "") + " split " + std::to_string(tc.nsplit) + "]";
             c->note(launch_gemm(p, epi, tc.tile, s), what);
         }
     }
