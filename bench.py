@@ -112,6 +112,50 @@ def bench_transforms(args, dev):
     print(json.dumps(result))
 
 
+def vendor_gemm(dev):
+    """torch.matmul (hipBLASLt / rocBLAS) against this library's GEMM on the same shapes and the same box.  A comparator for the
+    roofline fractions only: nothing in the product calls a library GEMM."""
+    import ctypes
+    import torch
+    import rtvla_capi as capi
+    lib, P = capi.load(), ctypes.c_void_p
+    shapes = [(788, 2048, 32768, "prefix gate+up as one GEMM (the library fuses GELU(gate) * up: N = 2 x 16384)"), (788, 2048, 16384, "prefix gate alone"),
+              (788, 16384, 2048, "prefix down"), (788, 2048, 2560, "prefix qkv"), (768, 1152, 3456, "SigLIP qkv"), (768, 1152, 4304, "SigLIP up"),
+              (768, 4304, 1152, "SigLIP down"), (8115, 1024, 4096, "DM0 ViT up-projection"), (8115, 4096, 1024, "DM0 ViT projection"),
+              (8115, 1024, 3072, "DM0 ViT qkv"), (51, 1024, 8192, "action-expert gate+up (M = 51)")]
+    st = torch.cuda.Stream()
+    rows = []
+    for M, K, N, what in shapes:
+        x = torch.randn(M, K, device=dev).bfloat16(); w = (torch.randn(K, N, device=dev) * 0.05).bfloat16()
+        out = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+        for _ in range(5):
+            torch.matmul(x, w, out=out)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(20):
+                torch.matmul(x, w, out=out)
+        g.replay(); torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(); g.replay(); e1.record(); torch.cuda.synchronize()
+        vendor_us = e0.elapsed_time(e1) * 1e3 / 20
+        mine = None
+        for tile, ns in ((capi.TILE_SKINNY, 1),) if M <= 64 else ((capi.TILE_AUTO, 1), (capi.TILE_AUTO, 0)):
+            need = lib.rtvla_linear_workspace_bytes(M, K, N, tile, ns)
+            if not need:
+                continue
+            ws = torch.empty(need, dtype=torch.uint8, device=dev)
+            ms = ctypes.c_float()
+            with torch.cuda.stream(st):
+                rc = lib.rtvla_time_linear(P(x.data_ptr()), M, K, P(w.data_ptr()), N, P(out.data_ptr()), P(ws.data_ptr()), need, tile, ns, 20, P(st.cuda_stream), ctypes.byref(ms))
+            torch.cuda.synchronize()
+            if rc == 0 and (mine is None or ms.value * 1e3 < mine):
+                mine = ms.value * 1e3
+        rows.append({"gemm": what, "M": M, "K": K, "N": N, "vendor_us": round(vendor_us, 1), "vendor_tflops": round(2.0 * M * K * N / vendor_us / 1e6),
+                     "rtvla_linear_us": round(mine, 1) if mine else None, "rtvla_tflops": round(2.0 * M * K * N / mine / 1e6) if mine else None})
+    print(json.dumps({"vendor_gemm": rows, "rtvla_version": lib.rtvla_version()}))
+
+
 def bench_dm0(args, dev, desc, views, lang, chunk):
     """The reference's third model at its own benchmark shape (/root/reference/benchmark.py:61-62, README.md:35)."""
     import torch
@@ -215,6 +259,9 @@ def main():
                          "and cold), measured in temporary graphs, and exit.  With a tuning build of the library (build.py -DRTVLA_TUNING, "
                          "selected by RTVLA_LIBRARY) --knockouts repeats the action-expert timings with parts of the kernels switched off")
     ap.add_argument("--knockouts", default="", help="comma-separated RTVLA_KO masks for --launch-times (tuning builds only)")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="comparator, not part of the product: time torch.matmul (the vendor GEMM library) on the GEMM shapes of the "
+                         "three models, 20 launches in a graph each, and the library's own kernel for the same shape through rtvla_time_linear")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: launch the roofline kernel a few times, then a "
                          "plain 256 MiB device copy whose counter reading calibrates the unit, and exit")
@@ -233,6 +280,8 @@ def main():
     seed = 1234
     if args.transforms:
         return bench_transforms(args, dev)
+    if args.vendor_gemm:
+        return vendor_gemm(dev)
     if model_name == "dm0":
         return bench_dm0(args, dev, desc, views, prompt, chunk)
     if model_name == "pi0":
