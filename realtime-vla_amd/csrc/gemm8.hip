@@ -197,7 +197,7 @@ RTVLA_DEVICE void gemm8_block(const GemmP& p, unsigned char* smem_raw, int m0, i
 }
 
 template <int MT, int EPI, bool MIXED>
-__global__ __launch_bounds__(512)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MT <= 4 ? 4 : 2, MT <= 4 ? 4 : 2)))
 void gemm8_kernel(GemmP p, int m_blocks, int n_blocks, int stages_total, int stages_per_split, int n_big) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int total = m_blocks * n_blocks * p.nsplit;
