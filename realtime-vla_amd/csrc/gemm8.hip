@@ -120,6 +120,66 @@ RTVLA_DEVICE void gemm8_block(const GemmP& p, unsigned char* smem_raw, int m0, i
         }
     }
 
+    if constexpr (EPI == EPI_VIT_QKV_ROPE) {
+        // DM0 ViT (dm0_infer.py:589-598), as in the four-wave kernel: + fp32 bias, rounded to bf16, 2-D rotary embedding on Q and
+        // K, per (image, head) Q and K as fragment-tiled [seq_pad][64] (16-byte pieces after a half swap between lane pairs),
+        // V^T transposed through a wave-private 2.3 KB of LDS into whole pieces of the permuted-key fragments
+#pragma unroll
+        for (int k = 0; k < MTW; ++k) {
+            const int m = m0 + (i0 + k) * 32 + r;
+            if (k >= mtw || m0 + (i0 + k) * 32 >= p.M) continue;
+            const int img = m / p.seq_pad, tok = m - img * p.seq_pad;
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const int nt0 = tile_of[j] * 32;
+                if (nt0 >= p.N16 * 16) continue;
+                const int which = nt0 >> 10, head = (nt0 & 1023) >> 6, d0 = nt0 & 63;
+                const size_t vh = (size_t)(img * 16 + head);
+                uint2 qk[4];
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    const int n0 = nt0 + 8 * grp + 4 * h;
+                    f32x4 v = {acc[k][j][4 * grp], acc[k][j][4 * grp + 1], acc[k][j][4 * grp + 2], acc[k][j][4 * grp + 3]};
+                    v += *(const f32x4*)(p.bias_f32 + n0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = round_bf16(v[e]);
+                    if (which < 2) {
+                        const bf16x4 cs = load4(p.rope + (size_t)min(tok, p.seq - 1) * 64 + d0 + 8 * grp + 4 * h);
+                        const float c0 = bf2f(cs[0]), s0 = bf2f(cs[1]), c1 = bf2f(cs[2]), s1 = bf2f(cs[3]);
+                        const f32x4 w = v;
+                        v[0] = w[0] * c0 - w[1] * s0; v[1] = w[1] * c0 + w[0] * s0;
+                        v[2] = w[2] * c1 - w[3] * s1; v[3] = w[3] * c1 + w[2] * s1;
+                        const bf16x4 pk = pack4(v);
+                        qk[grp] = *(const uint2*)&pk;
+                    } else {
+                        volatile bf16_t* tb = (volatile bf16_t*)(smem_raw + wave * 2304);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) tb[(8 * grp + 4 * h + e) * 36 + r] = f2bf(v[e]);
+                    }
+                }
+                if (which < 2) {
+                    bf16_t* const dst = (which == 0 ? p.q : p.k) + vh * ((size_t)p.seq_pad * 64);
+#pragma unroll
+                    for (int pr = 0; pr < 2; ++pr) {
+                        const uint2 keep = h ? qk[2 * pr + 1] : qk[2 * pr], send = h ? qk[2 * pr] : qk[2 * pr + 1];
+                        const uint2 recv = {(unsigned)__shfl_xor((int)send.x, 32, 64), (unsigned)__shfl_xor((int)send.y, 32, 64)};
+                        *(uint4*)(dst + ft_index(tok, d0 + 8 * (2 * pr + h), 2)) = h ? uint4{recv.x, recv.y, keep.x, keep.y} : uint4{keep.x, keep.y, recv.x, recv.y};
+                    }
+                } else {
+                    const int tok0 = tok - r;
+                    const int gq = lane >> 4, rq = lane & 15;
+#pragma unroll
+                    for (int dt = 0; dt < 2; ++dt) {
+                        const volatile uint2* src = (const volatile uint2*)(smem_raw + wave * 2304 + (16 * dt + rq) * 72 + gq * 8);
+                        const uint2 lo = {src[0].x, src[0].y}, hi = {src[4].x, src[4].y};
+                        const size_t frag = (size_t)(((d0 >> 4) + dt) * (p.seq_pad >> 5) + (tok0 >> 5)) * 64 + lane;
+                        *(uint4*)(p.vt + vh * ((size_t)64 * p.seq_pad) + frag * 8) = uint4{lo.x, lo.y, hi.x, hi.y};
+                    }
+                }
+            }
+        }
+        return;
+    }
     // ---- epilogue: lane (h, r) holds rows m0 + 32 (i0 + i) + r, columns 32 tile + 8 grp + 4 h + e.  The k-th row tiles of
     // the two wave halves are converted into two LDS tiles and copied out together as 16-byte chunks of row segments.
     constexpr int ESZ = (EPI == EPI_PARTIAL) ? 4 : 2;
@@ -260,6 +320,7 @@ int launch_gemm8(const GemmP& p, int epi, int tile, hipStream_t s) {
         case EPI_GEGLU:     return launch8_epi<EPI_GEGLU>(p, tile, s);
         case EPI_PARTIAL:   return launch8_epi<EPI_PARTIAL>(p, tile, s);
         case EPI_SWIGLU:    return launch8_epi<EPI_SWIGLU>(p, tile, s);
+        case EPI_VIT_QKV_ROPE: return launch8_epi<EPI_VIT_QKV_ROPE>(p, tile, s);
     }
     return 2;
 }

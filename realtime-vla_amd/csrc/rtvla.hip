@@ -121,7 +121,7 @@ constexpr int64_t ATTN_PARTIAL_FLOATS = 32 * 16 * (16 * 64 * 4 + 32);   // 32 ro
 // workgroup); tiles of 64 rows run two workgroups per CU, which then share the MFMA pipe but overlap
 // their load latency; all workgroups together cannot pull more than ~20 TB/s out of L2; every launch pays a
 // fixed ramp and an epilogue that grows with the tile; split-K adds the reduce pass over the fp32 partials.
-TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what, bool plain = false) {
+TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what, int eight = 0) {
     static const int tiles[] = {TILE_224x256, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};
     static const int splits[] = {1, 2, 3, 4, 6, 8};
 #ifdef RTVLA_TUNING
@@ -135,7 +135,8 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
 #endif
     // measured (M = 8115, K = 1024, N = 4096, bias + GELU): the eight-wave 256 x 256 tile takes 84-89 us where the best four-wave
     // tile takes 98-101 us; with 788 rows, with the gated epilogues and with fp32 split-K partials the four-wave tiles win
-    if (plain && M >= 4096 && stages <= 32 && ncols16 >= 128) return TileChoice{TILE8_256x256, 1};      // plain: bias (+ GELU) epilogue
+    // (eight: 1 = bias (+ GELU) epilogue, 2 = the ViT QKV epilogue, measured 75 us with the eight-wave 128 x 256 tile against 93 us)
+    if (eight && M >= 4096 && stages <= 32 && ncols16 >= 128) return TileChoice{eight == 1 ? TILE8_256x256 : TILE8_128x256, 1};
     double best = 1e30; TileChoice bc{TILE_128x256, 1};
     for (int tile : tiles) {
         const int bm = gemm_tile_bm(tile);
@@ -444,7 +445,7 @@ struct Sched {
         GemmP p = extra;
         p.A = A; p.lda = lda; p.a_rows = a_rows; p.M = M; p.B0 = B0; p.B1 = B1;
         p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.bgroup = bgroup;
-        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU || epi == EPI_SWIGLU, epi == EPI_PARTIAL, what, epi == EPI_BIAS || epi == EPI_BIAS_GELU);
+        const TileChoice tc = choose_tile(M, p.N16, p.K32p / 2, epi == EPI_GEGLU || epi == EPI_SWIGLU, epi == EPI_PARTIAL, what, (epi == EPI_BIAS || epi == EPI_BIAS_GELU) ? 1 : epi == EPI_VIT_QKV_ROPE ? 2 : 0);
         p.nsplit = tc.nsplit;
         if (epi == EPI_PARTIAL) {
             p.partial = c->B<float>("splitk_partial"); p.ldp = N; p.pstride = (size_t)M * N;
