@@ -81,7 +81,7 @@ enum rtvla_stage {
 
 /* Library version (no reference counterpart): raised whenever a kernel or the schedule changes, so that a
  * measurement recorded for one version is not mistaken for the current kernels. */
-#define RTVLA_VERSION 5
+#define RTVLA_VERSION 6
 int rtvla_version(void);
 
 /* Create a context for one shape set.  Replaces the tensor allocation block of
@@ -133,8 +133,10 @@ int rtvla_buffer_info(const rtvla_ctx* ctx, int index, const char** name, size_t
                       int64_t* rows, int64_t* cols, int64_t* ld, int32_t* elem_bytes);
 
 /* One-time device work after all weights are bound: re-tile weights into MFMA fragment order,
- * clear the workspace, Pi05: scale the output projection by -1/num_steps and compute the
- * time-conditioning style vectors (pi05_infer.py:669-722).  Enqueued on `hip_stream` (a
+ * clear the workspace, Pi05: scale the output projection by -1/num_steps, compute the
+ * time-conditioning style vectors (pi05_infer.py:669-722) and fold each (flow step, layer)'s adaptive RMS norm
+ * (pi05_infer.py:127-195) into a row-scaled copy of the weights that consume it plus an fp32 per-column term
+ * (num_steps x layers copies of the action expert's QKV / gate / up weights: 3.96 GB at full size).  Enqueued on `hip_stream` (a
  * hipStream_t passed as void*); the caller synchronises. */
 int rtvla_prepare(rtvla_ctx* ctx, void* hip_stream);
 

@@ -33,7 +33,10 @@ static inline size_t tiled_elems(int K, int N, int G = 1) { return (size_t)((n16
 // W[kb*16 + 8 (l >> 5) + j][nb*32 + (l & 31)], stored [nb / G][kb][nb % G] with the same K padding.
 static inline size_t tiled_elems_wide(int K, int N, int G) { return (size_t)(((N + 31) / 32 + G - 1) / G) * G * k32_padded(K) * 2 * 512; }
 
-void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide, hipStream_t s);
+// rowscale (optional, K values): row k of W is multiplied by 1 + rowscale[k] before the rounding to bf16
+void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide, hipStream_t s, const bf16_t* rowscale = nullptr);
+// out[n] = sum_k v[k] W[k][n] in fp32 (one-time work at prepare)
+void launch_vec_mat(const bf16_t* v, const bf16_t* W, int K, int N, float* out, hipStream_t s);
 void launch_pretile_padded(const bf16_t* W, int K, int K_pad, int N, bf16_t* out, hipStream_t s);
 
 // ----- large-M MFMA GEMM --------------------------------------------------------------
@@ -110,6 +113,8 @@ struct SkinnyP {
     int factor_f32;                            // SN_RMS: keep the row factor in fp32 (DM0) instead of rounding it to bf16 (Pi0)
     bf16_t* out; int ldo;
     const bf16_t* bias; const bf16_t* gate;    // per-column
+    const float* col_bias0; const float* col_bias1;   // SN_RMS with SK_QKV_ROPE / SK_GEGLU: fp32 per-column terms added after the row factor
+                                               // (Pi05: the shift of the adaptive RMS norm times the weights, see Sched::prepare)
     const bf16_t* rope;                        // [row][256]
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt; int kv_row0;
     RTVLA_KO_FIELD

@@ -6,7 +6,8 @@ namespace {
 
 // ---------------------------------------------------------------------------------------------
 // W[K][N] -> MFMA fragment tiles [nb][kb][lane][8] (see kernels.h)
-__global__ void pretile_kernel(const bf16_t* __restrict__ W, int K, int N, bf16_t* __restrict__ out, int KBp, int G, int wide, size_t chunks) {
+__global__ void pretile_kernel(const bf16_t* __restrict__ W, int K, int N, bf16_t* __restrict__ out, int KBp, int G, int wide, size_t chunks,
+                               const bf16_t* __restrict__ rowscale) {
     const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= chunks) return;
     const int lane = (int)(c & 63);
@@ -21,6 +22,7 @@ __global__ void pretile_kernel(const bf16_t* __restrict__ W, int K, int N, bf16_
     for (int j = 0; j < 8; ++j) {
         const int k = k0 + j;
         v[j] = (n < N && k < K) ? W[(size_t)k * N + n] : (bf16_t)0.0f;
+        if (rowscale && k < K) v[j] = f2bf(bf2f(v[j]) * (1.0f + bf2f(rowscale[k])));
     }
     *(bf16x8*)(out + c * 8) = v;
 }
@@ -197,17 +199,28 @@ __global__ void scale_kernel(bf16_t* p, size_t n, float f) {
 
 }  // namespace
 
-void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide, hipStream_t s) {
+void launch_pretile(const bf16_t* W, int K, int N, bf16_t* out, int G, int wide, hipStream_t s, const bf16_t* rowscale) {
     const int KBp = wide ? k32_padded(K) * 2 : k32_padded(K);
     const size_t chunks = (wide ? tiled_elems_wide(K, N, G) : tiled_elems(K, N, G)) / 8;
-    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, KBp, G, wide, chunks);
+    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, KBp, G, wide, chunks, rowscale);
+}
+
+__global__ void vec_mat_kernel(const bf16_t* __restrict__ v, const bf16_t* __restrict__ W, int K, int N, float* __restrict__ out) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k) acc += bf2f(v[k]) * bf2f(W[(size_t)k * N + n]);
+    out[n] = acc;
+}
+void launch_vec_mat(const bf16_t* v, const bf16_t* W, int K, int N, float* out, hipStream_t s) {
+    hipLaunchKernelGGL(vec_mat_kernel, dim3((N + 127) / 128), dim3(128), 0, s, v, W, K, N, out);
 }
 
 // W has K rows; the tiles are laid out as for K_pad rows (a multiple of 128), the rows past K zero: for a kernel that only takes
 // the padded K
 void launch_pretile_padded(const bf16_t* W, int K, int K_pad, int N, bf16_t* out, hipStream_t s) {
     const size_t chunks = tiled_elems(K_pad, N, 1) / 8;
-    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, k32_padded(K_pad), 1, 0, chunks);
+    hipLaunchKernelGGL(pretile_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, W, K, N, out, k32_padded(K_pad), 1, 0, chunks, (const bf16_t*)nullptr);
 }
 
 template <int NORM>

@@ -279,6 +279,12 @@ int build_tables(rtvla_ctx* c) {
         c->add_tiled("t_decoder_pre_attn_norm_mod_w", 1024, 3072, L);
         c->add_tiled("t_decoder_pre_ffn_norm_mod_w", 1024, 3072, L);
         c->add_tiled("t_decoder_final_norm_mod_w", 1024, 3072, 1);
+        // The adaptive RMS norm folded into its consumers: with y = x f (1 + scale) + shift (f the row's RMS factor),
+        // y W = f (x diag(1 + scale) W) + shift W.  Per (flow step, layer) the row-scaled weights are tiled once at prepare and
+        // shift W becomes an fp32 per-column term, so that the action-expert kernels run the same post-scaled product as Pi0's.
+        c->add_tiled("t_decoder_attn_qkv_ada", 1024, 2560, d.num_steps * L);
+        c->add_tiled("t_decoder_ffn_gate_ada", 1024, 4096, d.num_steps * L);
+        c->add_tiled("t_decoder_ffn_up_ada", 1024, 4096, d.num_steps * L);
         c->add_buf("decoder_out_proj_w_scaled", 1024, 32, 32);
         c->add_buf("decoder_out_proj_b_scaled", 1, 32, 32);
     }
@@ -309,6 +315,9 @@ int build_tables(rtvla_ctx* c) {
         c->add_buf("decoder_style_attn", d.num_steps, L * 3072, L * 3072);
         c->add_buf("decoder_style_ffn", d.num_steps, L * 3072, L * 3072);
         c->add_buf("decoder_style_final", d.num_steps, 3072, 3072);
+        c->add_buf("decoder_ada_bias_qkv", d.num_steps * L, 2560, 2560, 4);      // fp32: shift W per (step, layer)
+        c->add_buf("decoder_ada_bias_gate", d.num_steps * L, 4096, 4096, 4);
+        c->add_buf("decoder_ada_bias_up", d.num_steps * L, 4096, 4096, 4);
     }
     const int64_t pmax = std::max(S_v * 1152, S_e * 2048) * 8;
     c->add_buf("splitk_partial", 1, pmax, pmax, 4);
@@ -583,6 +592,11 @@ struct Sched {
         const bf16_t* st_attn = pi05 ? c->B("decoder_style_attn") + ((size_t)t * L + i) * 3072 : nullptr;
         const bf16_t* st_ffn = pi05 ? c->B("decoder_style_ffn") + ((size_t)t * L + i) * 3072 : nullptr;
         SkinnyP q = tiled_io(); q.rope = c->W("decoder_rope_weights"); q.q = c->B("decoder_q_buf"); q.k = Kc(i); q.vt = Vt(i); q.ldvt = c->keys_pad; q.kv_row0 = S_e;
+        if (pi05) {                                                  // adaptive RMS folded into the weights of this (step, layer)
+            const size_t tl = (size_t)t * L + i;
+            q.factor_f32 = 1; q.col_bias0 = c->B<float>("decoder_ada_bias_qkv") + tl * 2560;
+            skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_attn_qkv_ada", (int)tl), nullptr, 1024, 2560, SN_RMS, nullptr, SK_QKV_ROPE, q, "suffix qkv");
+        } else
         skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_attn_qkv_w", i), nullptr, 1024, 2560, norm, st_attn, SK_QKV_ROPE, q, "suffix qkv");
         AttnP a{};
         a.q = c->B("decoder_q_buf"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
@@ -593,6 +607,11 @@ struct Sched {
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
         skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
         SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 4096;
+        if (pi05) {
+            const size_t tl = (size_t)t * L + i;
+            g.factor_f32 = 1; g.col_bias0 = c->B<float>("decoder_ada_bias_gate") + tl * 4096; g.col_bias1 = c->B<float>("decoder_ada_bias_up") + tl * 4096;
+            skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_ffn_gate_ada", (int)tl), c->TW("t_decoder_ffn_up_ada", (int)tl), 1024, 4096, SN_RMS, nullptr, SK_GEGLU, g, "suffix geglu");
+        } else
         skinny(c->B("decoder_x"), 1024, S_d, c->TW("t_decoder_ffn_gate_w", i), c->TW("t_decoder_ffn_up_w", i), 1024, 4096, norm, st_ffn, SK_GEGLU, g, "suffix geglu");
         SkinnyP dn = tiled_io(); dn.out = c->B("decoder_x"); dn.ldo = 1024; dn.gate = pi05 ? st_ffn + 2048 : nullptr;
         skinny(c->B("decoder_hidden"), 4096, S_d, c->TW("t_decoder_ffn_down_w", i), nullptr, 4096, 1024, SN_NONE, nullptr, SK_RES, dn, "suffix down");
@@ -895,6 +914,24 @@ struct Sched {
         }
         SkinnyP f{}; f.a_tiled = 1; f.ldo = 3072; f.out = c->B("decoder_style_final"); f.bias = c->W("decoder_final_norm_mod_b");
         skinny(c->B("decoder_time_emb"), 1024, T, c->TW("t_decoder_final_norm_mod_w"), nullptr, 1024, 3072, SN_NONE, nullptr, SK_BIAS, f, "style final");
+        // the adaptive RMS norm of every (step, layer) folded into its consumers' weights: style = [scale | shift | gate]
+        for (int t = 0; t < T; ++t)
+            for (int i = 0; i < L; ++i) {
+                const size_t tl = (size_t)t * L + i;
+                const bf16_t* sa = c->B("decoder_style_attn") + tl * 3072;
+                const bf16_t* sf = c->B("decoder_style_ffn") + tl * 3072;
+                const bf16_t* wq = c->W("decoder_attn_qkv_w", (size_t)1024 * 2560, i);
+                const bf16_t* wg = c->W("decoder_ffn_gate_w", (size_t)1024 * 4096, i);
+                const bf16_t* wu = c->W("decoder_ffn_up_w", (size_t)1024 * 4096, i);
+                if (!tiles_loaded) {
+                    launch_pretile(wq, 1024, 2560, c->TW("t_decoder_attn_qkv_ada", (int)tl), 1, 0, s, sa);
+                    launch_pretile(wg, 1024, 4096, c->TW("t_decoder_ffn_gate_ada", (int)tl), 1, 0, s, sf);
+                    launch_pretile(wu, 1024, 4096, c->TW("t_decoder_ffn_up_ada", (int)tl), 1, 0, s, sf);
+                }
+                launch_vec_mat(sa + 1024, wq, 1024, 2560, c->B<float>("decoder_ada_bias_qkv") + tl * 2560, s);
+                launch_vec_mat(sf + 1024, wg, 1024, 4096, c->B<float>("decoder_ada_bias_gate") + tl * 4096, s);
+                launch_vec_mat(sf + 1024, wu, 1024, 4096, c->B<float>("decoder_ada_bias_up") + tl * 4096, s);
+            }
     }
 };
 

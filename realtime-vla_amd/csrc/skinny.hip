@@ -74,6 +74,7 @@ void skinny_kernel(SkinnyP p) {
     // what the epilogue will need from memory (old residual, RoPE pair, bias, gate) is requested now as well, by the
     // waves that will finish a row tile, so that no memory round trip is left after the reduction
     bf16x4 pre_old = {}, pre_cs = {}, pre_bias = {}, pre_gate = {};
+    f32x4 pre_cb0 = {0.f, 0.f, 0.f, 0.f}, pre_cb1 = {0.f, 0.f, 0.f, 0.f};
     if (w < SK_MTS) {
         const int me = min(m_base + w * 16 + r, p.M - 1);
         const int ne = tile * 16 + 4 * g;
@@ -85,6 +86,10 @@ void skinny_kernel(SkinnyP p) {
             pre_bias = load4(p.bias + ne);
         } else if constexpr (EPI == SK_QKV_ROPE) {
             if (ne < 2304) pre_cs = load4(p.rope + (size_t)me * 256 + (ne & 255));
+        }
+        if constexpr (NORM == SN_RMS && (EPI == SK_QKV_ROPE || EPI == SK_GEGLU)) {
+            if (p.col_bias0) pre_cb0 = *(const f32x4*)(p.col_bias0 + ne);
+            if (p.col_bias1) pre_cb1 = *(const f32x4*)(p.col_bias1 + ne);
         }
     }
     // keep every load above in flight before anything waits on one of them
@@ -176,6 +181,10 @@ void skinny_kernel(SkinnyP p) {
         if (!p.factor_f32) f = round_bf16(f);                            // the Pi0 reference keeps the factor in bf16, DM0 in fp32
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) v[nb] *= f;
+        if constexpr (EPI == SK_QKV_ROPE || EPI == SK_GEGLU) {
+            v[0] += pre_cb0;
+            if constexpr (NB == 2) v[1] += pre_cb1;
+        }
     }
     if (m >= p.M) return;
     const int n0 = tile * 16 + 4 * g;
@@ -248,9 +257,7 @@ int launch_skinny(const SkinnyP& p, int epi, hipStream_t s) {
     if (p.norm == SN_ADARMS && !p.style) return 1;
 #define SK_CASE(NCH_, NORM_, EPI_, MTS_) if (nch == NCH_ && p.norm == NORM_ && epi == EPI_) return launch_inst<NCH_, NORM_, EPI_, MTS_>(p, s)
     SK_CASE(1, SN_RMS, SK_QKV_ROPE, 4);
-    SK_CASE(1, SN_ADARMS, SK_QKV_ROPE, 4);
     SK_CASE(1, SN_RMS, SK_GEGLU, 4);
-    SK_CASE(1, SN_ADARMS, SK_GEGLU, 4);
     SK_CASE(1, SN_RMS, SK_SWIGLU, 4);
     SK_CASE(1, SN_NONE, SK_BIAS, 4);
     SK_CASE(1, SN_NONE, SK_BIAS_SILU, 4);
