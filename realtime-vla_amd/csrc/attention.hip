@@ -129,7 +129,7 @@ void mqa_kernel(AttnP p) {
 
     for (int kb = kb_begin + w; kb < kb_end; kb += WAVES) {
         const int key0 = kb * KBS;
-        const int kb_next = min(kb + WAVES, kb_end - 1);    // the last round re-reads a block instead of branching
+        const int kb_next = kb + WAVES;
         f32x4 st[MQ][NTK];
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
@@ -142,7 +142,7 @@ void mqa_kernel(AttnP p) {
 #pragma unroll
                 for (int mq = 0; mq < MQ; ++mq) st[mq][nt] = mfma16(kf[nt][kd], qf[mq][kd], st[mq][nt]);
         __builtin_amdgcn_sched_barrier(0);
-        load_k(kb_next);                                     // next block's K flies during softmax and P V
+        if (kb + WAVES < kb_end) load_k(kb_next);            // next block's K flies during softmax and P V (the suffix pass has one block per wave: nothing to fetch)
         __builtin_amdgcn_sched_barrier(0);
         bf16x8 pb[MQ][NTK / 2];
         bool full = key0 + KBS <= vis_lim;
@@ -210,7 +210,7 @@ void mqa_kernel(AttnP p) {
                 for (int mq = 0; mq < MQ; ++mq) o[mq][dt] = mfma16(vf[dt][kk], pb[mq][kk], o[mq][dt]);
             }
         __builtin_amdgcn_sched_barrier(0);
-        load_v(kb_next);
+        if (kb + WAVES < kb_end) load_v(kb_next);
         __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -259,6 +259,149 @@ void mqa_kernel(AttnP p) {
                 store4(attn_out_at(p, orow, dt * 16 + 4 * g), pack4(t * inv));
             }
         }
+    }
+}
+
+// Suffix pass with at most one 32-key block per wave (key splits of 128 keys): the four waves of a workgroup share the
+// PROBABILITIES instead of merging their outputs.  Wave w computes the logits of key block w (it alone reads that block
+// of K), the row maxima and then the probabilities are exchanged through LDS (16 floats and one 1 KB fragment per wave),
+// and every wave multiplies all four probability fragments with ITS quarter of the head width of V^T (16 / 4 d tiles x 4
+// key blocks: the same 16 fragments it would read of one key block), so each wave ends up with finished columns of the
+// partial and stores them straight to memory: no output exchange (64 KB each way), one barrier less.  Q is loaded once
+// per workgroup (each wave fetches a quarter) and shared through LDS.
+template <int HD>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+void suffix_attn_kernel(AttnP p) {
+    constexpr int KD = HD / 32, DT = HD / 16, DTW = DT / 4, QW = KD / 4;
+    static_assert(KD % 4 == 0, "Q fragments are dealt over four waves");
+    __shared__ bf16x8 qsh[KD][64];
+    __shared__ bf16x8 psh[4][64];
+    __shared__ float msh[4][16], lsh[4][16];
+    const int batch = blockIdx.y;
+    const bf16_t* const qbase = p.q + (size_t)batch * p.q_bstride;
+    const bf16_t* const kbase = p.k + (size_t)batch * p.k_bstride;
+    const bf16_t* const vbase = p.vt + (size_t)batch * p.vt_bstride;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int g = lane >> 4, r = lane & 15;
+    const int nsplit = p.nsplit_eff;
+    int rowblk, split;
+    if (nsplit == 1) { rowblk = blockIdx.x; split = 0; }
+    else {                                                               // all row blocks of one split on one XCD (see mqa_kernel)
+        const int spx = (nsplit + 7) >> 3;
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        split = xcd + 8 * (idx % spx); rowblk = idx / spx;
+        if (split >= nsplit) return;                                     // (whole workgroup, before any barrier)
+    }
+    const int m0 = rowblk * 16;
+    int vl = p.prefix_alloc;
+    if (p.valid_len) vl = max(0, min(*p.valid_len, p.prefix_alloc));
+    const int vis_lim = min(vl, p.keys);
+    const float sc2 = p.scale * 1.4426950408889634f;
+    const int nkb = (p.keys + 31) >> 5, keys32 = p.ldvt >> 5;
+    const int kb_begin = split * p.kb_per_split, kb_end = min(nkb, kb_begin + p.kb_per_split);
+    const int kb = kb_begin + w;
+    const bool have = kb < kb_end;                                       // (wave-uniform)
+
+    // everything this wave needs from memory, requested up front: its quarter of Q, its key block of K, its d tiles of V^T
+    bf16x8 qmine[QW];
+#pragma unroll
+    for (int i = 0; i < QW; ++i) qmine[i] = *(const bf16x8*)(qbase + ((size_t)(rowblk * KD + w * QW + i) * 64 + lane) * 8);
+    bf16x8 kf[2][KD];
+    if (have) {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kf[nt][kd] = *(const bf16x8*)(kbase + ((size_t)((kb * 2 + nt) * KD + kd) * 64 + lane) * 8);
+    }
+    bf16x8 vf[DTW][4];
+#pragma unroll
+    for (int i = 0; i < DTW; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)                                      // blocks past the end are clamped: their probabilities are zero
+            vf[i][j] = *(const bf16x8*)(vbase + ((size_t)((w * DTW + i) * keys32 + min(kb_begin + j, keys32 - 1)) * 64 + lane) * 8);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < QW; ++i) qsh[w * QW + i][lane] = qmine[i];
+    __syncthreads();
+
+    // ---- logits of this wave's key block, base-2 domain ----
+    f32x4 st[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    bool vis[2][4];
+    float mx = NEG_BIG;
+    const int row = m0 + r;
+    if (have) {
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const bf16x8 qf = qsh[kd][lane];
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) st[nt] = mfma16(kf[nt][kd], qf, st[nt]);
+        }
+        const int key0 = kb * 32;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int key = key0 + nt * 16 + 4 * g + v;
+                bool ok = key < p.keys;
+                if (key0 + 32 > vis_lim) {                               // (uniform) a block every row sees whole needs no mask arithmetic
+                    if (key < p.prefix_alloc) ok = ok && key < vl;
+                    else ok = ok && (row >= p.state_rows || key == p.prefix_alloc);
+                }
+                vis[nt][v] = ok;
+                const float sv = ok ? st[nt][v] * sc2 : NEG_BIG;
+                st[nt][v] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    } else {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) vis[nt][v] = false;
+    }
+    if (g == 0) msh[w][r] = mx;
+    __syncthreads();
+    const float mg = fmaxf(fmaxf(msh[0][r], msh[1][r]), fmaxf(msh[2][r], msh[3][r]));
+    float sum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float e = vis[nt][v] ? __builtin_amdgcn_exp2f(st[nt][v] - mg) : 0.f;
+            st[nt][v] = e;
+            sum += e;
+        }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    psh[w][lane] = cat44(pack4(st[0]), pack4(st[1]));
+    if (g == 0) lsh[w][r] = sum;
+    __syncthreads();
+
+    // ---- this wave's d tiles of O^T = V^T P^T over all four key blocks ----
+    bf16x8 pb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pb[j] = psh[j][lane];
+    const float lt = lsh[0][r] + lsh[1][r] + lsh[2][r] + lsh[3][r];
+    f32x4 o[DTW];
+#pragma unroll
+    for (int i = 0; i < DTW; ++i) {
+        o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[i] = mfma16(vf[i][j], pb[j], o[i]);
+    }
+    if (nsplit > 1) {
+        // partial record of one (row block, split): { O [DT][64] f32x4 | max [16] | sum [16] }, combined by attn_merge_kernel
+        constexpr int REC = DT * 64 * 4 + 32;
+        float* const mine = p.partial + (((size_t)batch * p.row_blocks + rowblk) * nsplit + split) * REC;
+#pragma unroll
+        for (int i = 0; i < DTW; ++i) *(f32x4*)(mine + ((w * DTW + i) * 64 + lane) * 4) = o[i];
+        if (w == 0 && g == 0) { mine[DT * 256 + r] = mg; mine[DT * 256 + 16 + r] = lt; }
+    } else if (row < p.rows) {
+        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+        const AttnOutRow orow = attn_out_row(p, batch, row, HD);
+#pragma unroll
+        for (int i = 0; i < DTW; ++i) store4(attn_out_at(p, orow, (w * DTW + i) * 16 + 4 * g), pack4(o[i] * inv));
     }
 }
 
@@ -410,6 +553,9 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
     }
     p.nsplit_eff = nsplit;
     p.row_blocks = blocks;
+    if (MQ == 1 && NTK == 2 && WAVES == 4 && !CAUSAL && p.kb_per_split <= 4)          // one key block per wave: the probability-sharing kernel
+        hipLaunchKernelGGL((suffix_attn_kernel<HD>), dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(256), 0, s, p);
+    else
     hipLaunchKernelGGL(kern, dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(WAVES * 64), smem, s, p);
     if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16, HD>), dim3(blocks * (HD / 64), p.batch), dim3(256), 0, s, p, nsplit);
     else if (nsplit > 1) hipLaunchKernelGGL((attn_merge_kernel<MQ, 8, HD>), dim3(blocks * (HD / 64), p.batch), dim3(256), 0, s, p, nsplit);
