@@ -467,19 +467,20 @@ int launch_epi(const GemmP& p, int tile, hipStream_t s) {
         case TILE_64x256:  return launch_cfg<4, 2, 2, EPI, false>(p, s);
         case TILE_64x128:  if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 2, 1, EPI, false>(p, s); else return 2;
         case TILE_128x128: if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 4, 1, EPI, false>(p, s); else return 2;
+        case TILE_96x128:  if constexpr (!EpiTraits<EPI>::dual) return launch_cfg<4, 3, 1, EPI, false>(p, s); else return 2;
     }
     return 2;
 }
 
 }  // namespace
 
-int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {224, 192, 160, 128, 64, 64, 128, 256, 224, 192, 128}; return v[tile]; }
-int gemm_tile_bn(int tile) { return (tile == TILE_64x128 || tile == TILE_128x128) ? 128 : 256; }
+int gemm_tile_bm(int tile) { static const int v[TILE_COUNT] = {224, 192, 160, 128, 64, 64, 128, 256, 224, 192, 128, 96}; return v[tile]; }
+int gemm_tile_bn(int tile) { return (tile == TILE_64x128 || tile == TILE_128x128 || tile == TILE_96x128) ? 128 : 256; }
 
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s) {
     if (p.M <= 0 || p.N16 <= 0 || p.K32p <= 0 || (p.K32p & 1) || p.a_rows <= 0 || p.bgroup < 1) return 1;
     if (epi != EPI_PARTIAL && p.nsplit > 1) return 1;
-    if (tile >= TILE8_256x256) return launch_gemm8(p, epi, tile, s);
+    if (gemm_tile_eight_waves(tile)) return launch_gemm8(p, epi, tile, s);
     switch (epi) {
         case EPI_BIAS:      return launch_epi<EPI_BIAS>(p, tile, s);
         case EPI_BIAS_GELU: return launch_epi<EPI_BIAS_GELU>(p, tile, s);

@@ -74,7 +74,9 @@ struct GemmP {
 // blocks cover ceil(M / 32) 32-row tiles exactly.
 enum GemmTile { TILE_224x256 = 0, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_64x128, TILE_128x128,
                 // the same 256-column tiles computed by eight waves (csrc/gemm8.hip), row-major epilogues only
-                TILE8_256x256, TILE8_224x256, TILE8_192x256, TILE8_128x256, TILE_COUNT };
+                TILE8_256x256, TILE8_224x256, TILE8_192x256, TILE8_128x256,
+                TILE_96x128, TILE_COUNT };
+inline bool gemm_tile_eight_waves(int tile) { return tile >= TILE8_256x256 && tile <= TILE8_128x256; }
 int gemm_tile_bm(int tile);
 int gemm_tile_bn(int tile);
 int launch_gemm(const GemmP& p, int epi, int tile, hipStream_t s);

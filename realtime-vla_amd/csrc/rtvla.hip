@@ -137,6 +137,18 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
     // tile takes 98-101 us; with 788 rows, with the gated epilogues and with fp32 split-K partials the four-wave tiles win
     // (eight: 1 = bias (+ GELU) epilogue, 2 = the ViT QKV epilogue, measured 75 us with the eight-wave 128 x 256 tile against 93 us)
     if (eight && M >= 4096 && stages <= 32 && ncols16 >= 128) return TileChoice{eight == 1 ? TILE8_256x256 : TILE8_128x256, 1};
+    // shapes where timing the launch inside a layer (weights streamed from HBM) disagrees with the model below: the K = 4304
+    // SigLIP down-projection gains from four K splits (more workgroups pulling the 9.9 MB of weights at once, 22.1 -> 19.3 us
+    // with the reduce pass at 768 rows, 20.4 -> 14.4 us at 256 rows), the 788-row prefix QKV from 96-row tiles (22.0 -> 20.5 us)
+    struct Measured { int ncols16, stages, splittable, m_lo, m_hi, tile, nsplit; };
+    static const Measured measured[] = {
+        {72, 68, 1, 1, 512, TILE_64x128, 4},
+        {72, 68, 1, 513, 768, TILE_128x128, 4},
+        {160, 32, 0, 769, 832, TILE_96x128, 1},
+    };
+    if (!dual)
+        for (const Measured& e : measured)
+            if (e.ncols16 == ncols16 && e.stages == stages && e.splittable == (splittable ? 1 : 0) && M >= e.m_lo && M <= e.m_hi) return TileChoice{e.tile, e.nsplit};
     double best = 1e30; TileChoice bc{TILE_128x256, 1};
     for (int tile : tiles) {
         const int bm = gemm_tile_bm(tile);
@@ -463,7 +475,7 @@ struct Sched {
         if (c->want(what)) {
             // the name a measurement reports carries the kernel variant: block tile and split-K factor
             c->last_name = std::string(what) + " [" + std::to_string(gemm_tile_bm(tc.tile)) + "x" + std::to_string(gemm_tile_bn(tc.tile)) +
-                           (tc.tile >= TILE8_256x256 ? " 8 waves" : "") + " split " + std::to_string(tc.nsplit) + "]";
+                           (gemm_tile_eight_waves(tc.tile) ? " 8 waves" : "") + " split " + std::to_string(tc.nsplit) + "]";
             c->note(launch_gemm(p, epi, tc.tile, s), what);
         }
     }
