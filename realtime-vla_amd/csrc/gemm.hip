@@ -276,8 +276,9 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
                 const int n = nbase + ch * (16 / ESZ);
                 if (mm < p.M && n < ncols && !KO(p, 8)) {                        // (KO 8: no global stores)
                     const uint4 val = *(const uint4*)(tbuf + row * ROWB + ch * 16);
-                    if constexpr (EPI == EPI_PARTIAL) *(uint4*)(p.partial + (size_t)split * p.pstride + (size_t)mm * p.ldp + n) = val;
-                    else *(uint4*)(p.out + (size_t)mm * p.ldo + n) = val;
+                    // (streaming hint: the output is read once by the next launch and should not displace the operand tiles in L2)
+                    if constexpr (EPI == EPI_PARTIAL) __builtin_nontemporal_store(*(const f32x4*)&val, (f32x4*)(p.partial + (size_t)split * p.pstride + (size_t)mm * p.ldp + n));
+                    else __builtin_nontemporal_store(*(const f32x4*)&val, (f32x4*)(p.out + (size_t)mm * p.ldo + n));
                 }
             }
           }
