@@ -366,6 +366,51 @@ def test_pi05_device_side_prompt_equals_host_staged_prompt():
         m_emb.forward_ids(img, noise, torch.zeros(3, dtype=torch.int64))
 
 
+def _word_tokenizer_dir(path):
+    """A local tokenizer directory AutoTokenizer can load offline: whitespace / punctuation split, one id per word of the
+    reference's prompt template and per state bin (stands in for the PaliGemma tokenizer, which does not ship here)."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    from transformers import PreTrainedTokenizerFast
+    words = ["[UNK]", "Task", ":", ",", ";", "State", "Action", "pick", "up", "the", "red", "cube"] + [str(i) for i in range(256)]
+    tok = Tokenizer(models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="[UNK]"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    PreTrainedTokenizerFast(tokenizer_object=tok, unk_token="[UNK]").save_pretrained(str(path))
+    return len(words)
+
+
+def test_pi05_discrete_state_prompt_through_a_tokenizer(tmp_path):
+    """discrete_state_input=True (pi05_infer.py:539-562, :769-785): the prompt template is tokenised on the host per call,
+    max_prompt_len comes from the longest prompt, and forward(images, noise, task_prompt, state_tokens) must equal (a) the
+    same ids handed to forward_ids, bit for bit, and (b) the CPU oracle fed with embedding[ids] * sqrt(2048)."""
+    import numpy as np
+    from pi05_infer import Pi05Inference
+    from oracle import pi05 as oracle_pi05
+    dev, views, chunk, state_dim = "cuda:0", 1, 10, 5
+    vocab = _word_tokenizer_dir(tmp_path)
+    ck = syn.pi05_checkpoint(33, 0, dev, 1, 2, state_tokens=0, norms="random")
+    del ck["language_embeds"]
+    ck["embedding_weight"] = syn.normal_bf16(33, "embedding_weight_words", (vocab, 2048), 0.02, dev)
+    img, _, noise = syn.observation(33, views, chunk, dev)
+    with pytest.raises(KeyError):                                         # the reference's check, pi05_infer.py:559-560
+        Pi05Inference({k: v for k, v in ck.items() if k != "embedding_weight"}, views, chunk, tokenizer_path=str(tmp_path))
+    m = Pi05Inference(ck, views, chunk, tokenizer_path=str(tmp_path), max_tokenize_len=64, discrete_state_input=True,
+                      max_prompt_text="pick_up the red cube", state_dim_for_max_prompt=state_dim)
+    # "Task : pick up the red cube , State : <5 bins> ; Action :" = 2 + 5 + 3 + 5 + 3 words
+    assert m.max_prompt_len == 18 and m.device_prompt
+    for prompt, bins in (("pick_up the red cube", np.array([3, 255, 17, 0, 128])), ("pick up", np.array([9, 8]))):
+        ids = m.build_prompt_ids(prompt, bins)
+        assert ids.dtype == torch.int64 and int(ids.max()) < vocab and (ids != 0).all()      # no unknown word
+        a = m.forward(img, noise, task_prompt=prompt, state_tokens=bins).float().clone()
+        b = m.forward_ids(img, noise, ids).float().clone()
+        torch.cuda.synchronize()
+        assert torch.equal(a, b)
+        embeds = (ck["embedding_weight"][ids.to(dev)].float() * (2048.0 ** 0.5)).to(torch.bfloat16).cpu()
+        ref = oracle_pi05.forward({k: v.cpu() for k, v in ck.items() if k != "embedding_weight"}, img.cpu(), noise.cpu(),
+                                  prompt_embeds=embeds.float(), max_prompt_len=m.max_prompt_len)
+        mae = (a.cpu() - ref.float()).abs().mean().item()
+        assert mae <= 1e-2, (prompt, mae)
+
+
 def test_constructor_errors_match_the_reference():
     from pi0_infer import Pi0Inference
     ck = syn.pi0_checkpoint(4, 1, "cuda:0", 1, 1)
