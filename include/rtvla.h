@@ -56,7 +56,7 @@ typedef struct rtvla_dims {
     int32_t num_views;       /* 1..4 camera views of 224x224x3 (DM0: images of 728x728)               */
     int32_t prompt_len;      /* Pi0: rows of language_embeds; Pi05: max_prompt_len (allocated rows);
                                 DM0: max_lang_len (token ids)                                          */
-    int32_t chunk_size;      /* action chunk; Pi0 suffix = chunk+1 rows, Pi05 / DM0 = chunk rows (<= 64) */
+    int32_t chunk_size;      /* action chunk; Pi0 suffix = chunk+1 rows, Pi05 / DM0 = chunk rows (Pi0 / Pi05: <= 128 rows, DM0: <= 64) */
     int32_t num_steps;       /* Euler flow steps (the reference hard-codes 10; Pi05 / DM0: at most 10) */
     int32_t vision_layers;   /* SigLIP layers (27); DM0: ViT layers (23)                               */
     int32_t llm_layers;      /* prefix layers == action-expert layers (18; DM0: 28)                    */

@@ -113,7 +113,7 @@ constexpr int PATCH_LD = 640;      // 588 patch features padded to a multiple of
 constexpr int VHID_LD = 4352;      // 4304 padded to a multiple of 64
 constexpr int XN_LD = 2048 + 64;   // row strides that are a large power of two put every row of a K stage on the same L2 channel
 constexpr int EHID_LD = 16384 + 64;
-constexpr int64_t ATTN_PARTIAL_FLOATS = 32 * 16 * (16 * 64 * 4 + 32);   // 32 row blocks x 16 key splits of the suffix attention
+constexpr int64_t ATTN_PARTIAL_FLOATS = 64 * 16 * (16 * 64 * 4 + 32);   // 64 row blocks (128 suffix rows x 8 heads) x 16 key splits of the suffix attention
 
 // Pick block tile and split-K factor from a cost model fitted to measurements on MI355X.  One K stage of a
 // workgroup takes the larger of its MFMA time (32 cycles per 32x32x16 MFMA at the ~2.05 GHz the chip sustains,
@@ -317,11 +317,12 @@ int build_tables(rtvla_ctx* c) {
     c->add_buf("encoder_hidden", S_e, 16384, EHID_LD);
     c->add_buf("encoder_K", L * c->keys_pad, 256, 256);           // fragment-tiled [keys_pad][256] per layer
     c->add_buf("encoder_Vt", L * 256, c->keys_pad, c->keys_pad);  // tiled V^T [256][keys_pad] per layer
-    c->add_buf("decoder_x", 64, 1024, 1024);                      // the decoder_* activations are fragment-tiled
-    c->add_buf("decoder_x_buf", 64, 1024, 1024);
-    c->add_buf("decoder_q_buf", 512, 256, 256);
-    c->add_buf("decoder_attn", 64, 2048, 2048);
-    c->add_buf("decoder_hidden", 64, 4096, 4096);
+    const int64_t Rd = ((S_d + 63) / 64) * 64;                    // suffix rows padded to the 64-row blocks of the action-expert kernels
+    c->add_buf("decoder_x", Rd, 1024, 1024);                      // the decoder_* activations are fragment-tiled
+    c->add_buf("decoder_x_buf", Rd, 1024, 1024);
+    c->add_buf("decoder_q_buf", 8 * Rd, 256, 256);
+    c->add_buf("decoder_attn", Rd, 2048, 2048);
+    c->add_buf("decoder_hidden", Rd, 4096, 4096);
     if (pi05) {
         c->add_buf("decoder_time_emb", 64, 1024, 1024);           // fragment-tiled, one row per step
         c->add_buf("decoder_style_attn", d.num_steps, L * 3072, L * 3072);
@@ -980,7 +981,7 @@ int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out) {
     if (d.num_views < 1 || d.num_views > 4 || d.prompt_len < 0 || d.chunk_size < 1 || d.num_steps < 1) return RTVLA_ERR_ARG;
     if (d.vision_layers < 1 || d.llm_layers < 1) return RTVLA_ERR_ARG;
     const int S_d = d.chunk_size + (d.model == RTVLA_PI0 ? 1 : 0);
-    if (S_d > 64) return RTVLA_ERR_LIMIT;
+    if (S_d > (d.model == RTVLA_DM0 ? 64 : 128)) return RTVLA_ERR_LIMIT;        // two 64-row blocks of the action-expert kernels (DM0's buffers hold one)
     if (d.model != RTVLA_PI0 && d.num_steps > 10) return RTVLA_ERR_LIMIT;       // the per-step time tables have 10 rows
     if (d.prompt_len > 4096) return RTVLA_ERR_LIMIT;
     rtvla_ctx* c = new (std::nothrow) rtvla_ctx();
@@ -1228,7 +1229,7 @@ int plan_linear(int M, int K, int N, int tile, int nsplit, LinearPlan* pl) {
     p.K128 = k32_padded(K) * 32;
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     if (p.skinny) {
-        if (M > 64 || (K != 1024 && K != 2048 && K != 4096) || nsplit > 1) return RTVLA_ERR_LIMIT;
+        if (M > 128 || (K != 1024 && K != 2048 && K != 4096) || nsplit > 1) return RTVLA_ERR_LIMIT;
         p.tile = tile; p.nsplit = 1;
         p.w_off = 0; p.bias_off = up(tiled_elems(K, N) * 2); p.total = p.bias_off + up((size_t)N * 2);
         *pl = p; return RTVLA_OK;

@@ -1,4 +1,4 @@
-// Weight-streaming GEMM for the action expert (M <= 64 rows), replacing the decoder-side Triton
+// Weight-streaming GEMM for the action expert (M <= 128 rows, in row blocks of 64 or 16), replacing the decoder-side Triton
 // kernels of /root/reference/pi0_infer.py:82-124, :693-725, :939-1039, :1122-1163 and
 // /root/reference/pi05_infer.py:22-64, :78-113, :127-195.
 //
@@ -248,7 +248,7 @@ int launch_inst(const SkinnyP& p, hipStream_t s) {
 }  // namespace
 
 int launch_skinny(const SkinnyP& p, int epi, hipStream_t s) {
-    if (p.M <= 0 || p.M > 64 || p.N16 <= 0) return 1;
+    if (p.M <= 0 || p.M > 128 || p.N16 <= 0) return 1;      // (the row blocks of blockIdx.y; the callers' buffers hold at most 128 rows)
     if (p.K != 1024 && p.K != 2048 && p.K != 4096) return 1;
     if (p.K32p < p.K / 32 || p.lda < p.K || (p.lda & 31)) return 1;
     if (p.out_tiled && (p.ldo & 31)) return 1;

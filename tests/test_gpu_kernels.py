@@ -82,7 +82,8 @@ def test_mfma_gemm_every_tile_and_split_against_fp32_matmul(M, K, N):
         assert res is not None and res[0] <= REL_TOL and res[1] <= 1.01, (nsplit, res)
 
 
-@pytest.mark.parametrize("M,K,N", [(51, 1024, 2560), (51, 2048, 1024), (51, 4096, 1024), (64, 1024, 4096), (1, 1024, 1024), (17, 2048, 48)])
+@pytest.mark.parametrize("M,K,N", [(51, 1024, 2560), (51, 2048, 1024), (51, 4096, 1024), (64, 1024, 4096), (1, 1024, 1024), (17, 2048, 48),
+                                   (101, 1024, 2560), (128, 4096, 1024), (65, 2048, 1024)])      # (the last three: two 64-row blocks / up to eight 16-row blocks)
 def test_weight_streaming_kernel_against_fp32_matmul(M, K, N):
     import rtvla_capi as capi
     lib = capi.load()
@@ -95,7 +96,7 @@ def test_unit_entry_rejects_what_it_cannot_run():
     lib = capi.load()
     assert lib.rtvla_linear_workspace_bytes(16, 12, 16, -1, 1) == 0          # K not a multiple of 8
     assert lib.rtvla_linear_workspace_bytes(16, 16, 24, -1, 1) == 0          # N not a multiple of 16
-    assert lib.rtvla_linear_workspace_bytes(65, 1024, 64, capi.TILE_SKINNY, 1) == 0
+    assert lib.rtvla_linear_workspace_bytes(129, 1024, 64, capi.TILE_SKINNY, 1) == 0
     assert lib.rtvla_linear_workspace_bytes(16, 512, 64, capi.TILE_SKINNY, 1) == 0
     assert lib.rtvla_linear_workspace_bytes(64, 128, 4096, 0, 2) == 0        # split-K rows wider than the reduce kernel takes
     x = torch.zeros(16, 128, dtype=torch.bfloat16, device="cuda:0")

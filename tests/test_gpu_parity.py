@@ -107,11 +107,11 @@ class Case:
     # ---- buffer access in the library's layouts ----
     def dec_x(self):
         from _engine import untile_ft
-        return untile_ft(self.B["decoder_x"], 64, 1024)[: self.S_d]
+        return untile_ft(self.B["decoder_x"], self.B["decoder_x"].numel() // 1024, 1024)[: self.S_d]
 
     def set_dec_x(self, x):
         from _engine import tile_ft
-        full = torch.zeros(64, 1024, dtype=torch.bfloat16, device="cuda")
+        full = torch.zeros(self.B["decoder_x"].numel() // 1024, 1024, dtype=torch.bfloat16, device="cuda")
         full[: self.S_d] = bf(x)
         self.B["decoder_x"].reshape(-1).copy_(tile_ft(full))
 
@@ -264,7 +264,9 @@ def test_pi0_two_views_ragged_prefix():
     ("pi0", 1, 1, 1, 0),        # one action row, one prompt token: 258 prefix rows, 2 suffix rows
     ("pi0", 3, 37, 33, 0),      # odd everything: 805 prefix rows (GEMM row tiles with a ragged tail), 34 suffix rows
     ("pi0", 2, 200, 50, 0),     # long prompt on two views: 712 prefix rows, 763 keys (6 key splits)
-    ("pi05", 2, 5, 64, 9),      # Pi05 at the 64-row limit of the action-expert tile
+    ("pi05", 2, 5, 64, 9),      # Pi05 with exactly one 64-row block of the action-expert kernels
+    ("pi0", 1, 3, 100, 0),      # 101 suffix rows: two 64-row blocks, 51 attention row blocks
+    ("pi05", 1, 5, 128, 4),     # Pi05 at the 128-row limit
     ("pi05", 3, 100, 7, 0),     # Pi05, long prompt, short chunk
 ])
 def test_shape_sweep_against_the_oracle(model, views, prompt, chunk, state_tokens):
@@ -422,7 +424,7 @@ def test_constructor_errors_match_the_reference():
     with pytest.raises(RuntimeError):
         Pi0Inference(dict(ck, vision_final_norm_w=torch.zeros(7)), 1, 10)
     with pytest.raises(RuntimeError):
-        Pi0Inference(ck, 1, 64)                                            # 65 suffix rows exceed the 64-row tile
+        Pi0Inference(ck, 1, 128)                                           # 129 suffix rows exceed the two 64-row blocks
     m = Pi0Inference(ck, 1, 10)
     with pytest.raises(RuntimeError):
         m.forward(torch.zeros(2, 224, 224, 3), torch.zeros(32), torch.zeros(10, 32))
