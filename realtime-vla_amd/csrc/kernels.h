@@ -127,6 +127,8 @@ int launch_skinny(const SkinnyP& p, int epi, hipStream_t s);
 // (`out` fragment-tiled with first row out_row0 when out_tiled)
 void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t* bias, bf16_t* out, int ldo,
                          int M, int K, int N, int act_silu, int out_tiled, int out_row0, hipStream_t s);
+struct SmallLinearJob { const bf16_t* x; int ldx; const bf16_t* W; const bf16_t* bias; bf16_t* out; int ldo; int M, K, N, act_silu, out_tiled, out_row0; };
+void launch_small_linear2(const SmallLinearJob& a, const SmallLinearJob& b, hipStream_t s);      // two independent jobs in one launch (b.M = 0: one)
 
 // ----- attention --------------------------------------------------------------------------
 struct AttnP {

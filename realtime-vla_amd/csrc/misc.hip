@@ -125,29 +125,32 @@ __global__ void im2col_kernel(const bf16_t* __restrict__ img, bf16_t* __restrict
 }
 
 // tiny-K linear: one thread per output element, W[K][N] row-major (coalesced over n)
-__global__ void small_linear_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ W,
-                                    const bf16_t* __restrict__ bias, bf16_t* __restrict__ out, int ldo,
-                                    int M, int K, int N, int act_silu, int out_tiled, int out_row0) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= M * N) return;
-    const int m = idx / N, n = idx - m * N;
-    float acc = bias ? bf2f(bias[n]) : 0.f;
-    if (K == 32) {
+RTVLA_DEVICE void small_linear_one(const SmallLinearJob& j, int idx) {
+    const int m = idx / j.N, n = idx - m * j.N;
+    float acc = j.bias ? bf2f(j.bias[n]) : 0.f;
+    if (j.K == 32) {
         // every operand is requested before the first use: a dependent load per k would cost 32 memory round trips
         bf16x8 xr[4];
         bf16_t wc[32];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) xr[q] = *(const bf16x8*)(x + (size_t)m * ldx + q * 8);
+        for (int q = 0; q < 4; ++q) xr[q] = *(const bf16x8*)(j.x + (size_t)m * j.ldx + q * 8);
 #pragma unroll
-        for (int k = 0; k < 32; ++k) wc[k] = W[(size_t)k * N + n];
+        for (int k = 0; k < 32; ++k) wc[k] = j.W[(size_t)k * j.N + n];
 #pragma unroll
         for (int k = 0; k < 32; ++k) acc += bf2f(xr[k >> 3][k & 7]) * bf2f(wc[k]);
     } else {
-        for (int k = 0; k < K; ++k) acc += bf2f(x[(size_t)m * ldx + k]) * bf2f(W[(size_t)k * N + n]);
+        for (int k = 0; k < j.K; ++k) acc += bf2f(j.x[(size_t)m * j.ldx + k]) * bf2f(j.W[(size_t)k * j.N + n]);
     }
-    if (act_silu) acc = siluf(acc);
-    if (out_tiled) out[ft_index(m + out_row0, n, ldo >> 5)] = f2bf(acc);
-    else out[(size_t)m * ldo + n] = f2bf(acc);
+    if (j.act_silu) acc = siluf(acc);
+    if (j.out_tiled) j.out[ft_index(m + j.out_row0, n, j.ldo >> 5)] = f2bf(acc);
+    else j.out[(size_t)m * j.ldo + n] = f2bf(acc);
+}
+// one launch for up to two independent tiny linears (the state-token and the action input projections of a flow step)
+__global__ void small_linear_kernel(SmallLinearJob a, SmallLinearJob b) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int na = a.M * a.N;
+    if (idx < na) small_linear_one(a, idx);
+    else if (idx - na < b.M * b.N) small_linear_one(b, idx - na);
 }
 
 __global__ void copy_rows_kernel(const bf16_t* __restrict__ src, int lds, bf16_t* __restrict__ dst, int ldd, int rows, int cols8) {
@@ -260,8 +263,14 @@ void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hi
 
 void launch_small_linear(const bf16_t* x, int ldx, const bf16_t* W, const bf16_t* bias, bf16_t* out, int ldo,
                          int M, int K, int N, int act_silu, int out_tiled, int out_row0, hipStream_t s) {
-    const int total = M * N;
-    hipLaunchKernelGGL(small_linear_kernel, dim3((total + 255) / 256), dim3(256), 0, s, x, ldx, W, bias, out, ldo, M, K, N, act_silu, out_tiled, out_row0);
+    SmallLinearJob j{x, ldx, W, bias, out, ldo, M, K, N, act_silu, out_tiled, out_row0};
+    launch_small_linear2(j, SmallLinearJob{}, s);
+}
+
+void launch_small_linear2(const SmallLinearJob& a, const SmallLinearJob& b, hipStream_t s) {
+    const int total = a.M * a.N + b.M * b.N;
+    if (total <= 0) return;
+    hipLaunchKernelGGL(small_linear_kernel, dim3((total + 255) / 256), dim3(256), 0, s, a, b);
 }
 
 void launch_copy_rows(const bf16_t* src, int lds, bf16_t* dst, int ldd, int rows, int cols, hipStream_t s) {

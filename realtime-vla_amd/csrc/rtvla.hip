@@ -577,16 +577,15 @@ struct Sched {
     void suffix_step_begin(int t) {
         const int ch = d.chunk_size;
         if (!pi05) {
-            // state token -> row 0 (re-projected every step: the residual stream is updated in place)
-            if (c->want("state proj")) {
-                launch_small_linear(c->W("observation_state_normalized"), 32, c->W("decoder_state_in_proj_w"), c->W("decoder_state_in_proj_b"),
-                                    c->B("decoder_x"), 1024, 1, 32, 1024, 0, 1, 0, s);
-                c->note(0, "state proj");
-            }
-            if (c->want("action in")) {
-                launch_small_linear(c->W("diffusion_noise"), 32, c->W("decoder_action_fused_in_proj_w"),
-                                    c->W("decoder_action_fused_time_biases", 1024, t % 10), c->B("decoder_x_buf"), 1024, ch, 32, 1024, 1, 1, 0, s);
-                c->note(0, "action in");
+            // state token -> row 0 of the residual stream (re-projected every step: the stream is updated in place) and the fused
+            // action/time input projection + SiLU -> decoder_x_buf, as ONE launch: the two are independent
+            if (c->want("state + action in")) {
+                SmallLinearJob st{c->W("observation_state_normalized"), 32, c->W("decoder_state_in_proj_w"), c->W("decoder_state_in_proj_b"),
+                                  c->B("decoder_x"), 1024, 1, 32, 1024, 0, 1, 0};
+                SmallLinearJob ai{c->W("diffusion_noise"), 32, c->W("decoder_action_fused_in_proj_w"), c->W("decoder_action_fused_time_biases", 1024, t % 10),
+                                  c->B("decoder_x_buf"), 1024, ch, 32, 1024, 1, 1, 0};
+                launch_small_linear2(st, ai, s);
+                c->note(0, "state + action in");
             }
             SkinnyP e = tiled_io(0, 1); e.out = c->B("decoder_x"); e.ldo = 1024; e.bias = c->W("decoder_action_mlp_b");
             skinny(c->B("decoder_x_buf"), 1024, ch, c->TW("t_decoder_action_mlp_w"), nullptr, 1024, 1024, SN_NONE, nullptr, SK_BIAS, e, "action mlp");
