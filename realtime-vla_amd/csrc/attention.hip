@@ -177,8 +177,7 @@ void mqa_kernel(AttnP p) {
                         mx = fmaxf(mx, s);
                     }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = rows_max(mx);
             if (__any(mx > mrun[mq])) {                       // the accumulator is rescaled only when some row's maximum grew
                 const float mnew = fmaxf(mrun[mq], mx);
                 const float alpha = __builtin_amdgcn_exp2f(mrun[mq] - mnew);
@@ -196,8 +195,7 @@ void mqa_kernel(AttnP p) {
                     st[mq][nt][v] = e;
                     sum += e;
                 }
-            sum += __shfl_xor(sum, 16, 64);
-            sum += __shfl_xor(sum, 32, 64);
+            sum = rows_sum(sum);
             lrun[mq] += sum;
 #pragma unroll
             for (int kk = 0; kk < NTK / 2; ++kk) pb[mq][kk] = cat44(pack4(st[mq][2 * kk]), pack4(st[mq][2 * kk + 1]));
@@ -352,8 +350,7 @@ void suffix_attn_kernel(AttnP p) {
                 st[nt][v] = sv;
                 mx = fmaxf(mx, sv);
             }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = rows_max(mx);
     } else {
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
@@ -372,8 +369,7 @@ void suffix_attn_kernel(AttnP p) {
             st[nt][v] = e;
             sum += e;
         }
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
+    sum = rows_sum(sum);
     psh[w][lane] = cat44(pack4(st[0]), pack4(st[1]));
     if (g == 0) lsh[w][r] = sum;
     __syncthreads();
@@ -498,8 +494,7 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
             for (int v = 0; v < 4; ++v) { st[nt][v] *= scale; mx = fmaxf(mx, st[nt][v]); }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = rows_max(mx);
         if (__any(mx > mrun)) {
             const float mnew = fmaxf(mrun, mx);
             const float alpha = __builtin_amdgcn_exp2f(mrun - mnew);
@@ -513,8 +508,7 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
             for (int v = 0; v < 4; ++v) { st[nt][v] = __builtin_amdgcn_exp2f(st[nt][v] - mrun); sum += st[nt][v]; }
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
+        sum = rows_sum(sum);
         lrun += sum;
         bf16x8 pb[2];
 #pragma unroll

@@ -68,8 +68,35 @@ RTVLA_DEVICE size_t vt_index(int d, int key, int keys32) {
     return ((size_t)((d >> 4) * keys32 + (key >> 5)) * 64 + (d & 15) + 16 * ((mm & 15) >> 2)) * 8 + 4 * (mm >> 4) + (mm & 3);
 }
 
+// Reductions across the four 16-lane rows of a wavefront (lanes that differ in bits 4 and 5) with gfx950's register-file
+// swaps instead of LDS permutes: v_permlane16_swap exchanges the odd rows of one register with the even rows of another,
+// v_permlane32_swap the upper half of one with the lower half of the other, so after swapping a value with its own copy
+// every lane holds its own and its partner's value in the two registers (a dependent ds_bpermute costs an LDS round trip).
+typedef unsigned rtvla_u2 __attribute__((ext_vector_type(2)));
+RTVLA_DEVICE float rows_max(float v) {
+    rtvla_u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+RTVLA_DEVICE float rows_sum(float v) {
+    rtvla_u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+RTVLA_DEVICE float halves_max(float v) {
+    const rtvla_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+RTVLA_DEVICE float halves_sum(float v) {
+    const rtvla_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 RTVLA_DEVICE float wave_sum(float v) {
+    v = rows_sum(v);
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    for (int o = 8; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
 }

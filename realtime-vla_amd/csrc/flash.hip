@@ -130,7 +130,7 @@ void flash_kernel(AttnP p, int items_per_batch, int batches_per_xcd) {
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[b][e]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = halves_max(mx);
         if (__any(mx > m)) {
             const float mnew = fmaxf(m, mx);
             const float alpha = __builtin_amdgcn_exp2f((m - mnew) * c);
@@ -159,7 +159,7 @@ void flash_kernel(AttnP p, int items_per_batch, int batches_per_xcd) {
         __syncthreads();
     }
 
-    l += __shfl_xor(l, 32, 64);
+    l = halves_sum(l);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     const int row = row0 + n;
     if (row < p.rows) {

@@ -111,8 +111,7 @@ void skinny_kernel(SkinnyP p) {
                         const bf16x2 x2 = {a[0][mt][i][j], a[0][mt][i][j + 1]};
                         s = __builtin_amdgcn_fdot2_f32_bf16(x2, x2, s, false);
                     }
-                s += __shfl_xor(s, 16, 64);
-                s += __shfl_xor(s, 32, 64);
+                s = rows_sum(s);
                 ss[mt] = s;
             }
             if (g == 0) {
