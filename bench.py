@@ -369,6 +369,12 @@ def main():
     assert geglu_name.startswith("prefix geglu"), geglu_name
     geglu_flop = 2.0 * 2.0 * S_e * 2048 * 16384
     mfma = geglu_flop / (geglu_ms * 1e-3) / 1e12
+    # bytes the launch pulls from L2 into the CUs, fixed by its block tile (no operand is reused out of L1): every column block
+    # reads the (32-row padded) activations once, every row block the gate and up weights once
+    import re
+    bm, bn = (int(v) for v in re.search(r"\[(\d+)x(\d+)", geglu_name).groups())
+    m_pad = 32 * ((S_e + 31) // 32)
+    l2_bytes = 2.0 * 2048 * ((2 * 16384 // bn) * m_pad + ((m_pad + bm - 1) // bm) * 2 * 16384)
     roofline = {"bound": "mfma", "kernel": "prefix GeGLU GEMM (gemm_mfma_kernel, EPI_GEGLU), M=%d K=2048 N=2x16384" % S_e,
                 "achieved": round(mfma, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(mfma / MFMA_PEAK_TFLOPS, 4),
                 "launch_ms": round(geglu_ms, 4), "launch_ms_cache_warm": round(geglu_warm_ms, 4),
@@ -376,7 +382,9 @@ def main():
                 # profiles/ for exactly this kernel variant and library version (null otherwise)
                 "traffic": profiled_traffic("gemm_geglu_%s_hbm_traffic.md" % PROFILE_TAGS.get(args.config), geglu_name, args.config, lib_version),
                 "kernel_variant": geglu_name,
-                "algorithmic_bytes": 2.0 * (S_e * 2048 + 2 * 2048 * 16384 + S_e * 16384)}
+                "algorithmic_bytes": 2.0 * (S_e * 2048 + 2 * 2048 * 16384 + S_e * 16384),
+                # informational: the rate at which the launch draws its operand tiles from L2 (the kernels here top out near 10 TB/s)
+                "l2_to_cu": {"bytes": l2_bytes, "tb_per_s": round(l2_bytes / (geglu_ms * 1e-3) / 1e12, 2)}}
     # the action-expert side: one suffix layer (5 launches) streams 18 D_L-sized weight sets per step
     layer_ms = ctx.time_stage(capi.STAGE_SUFFIX_LAYER, -1, 0, 5, stream)          # all 18 layers in turn: weights cold, as in the forward
     layer_warm_ms = ctx.time_stage(capi.STAGE_SUFFIX_LAYER, 3, 0, 20, stream)
