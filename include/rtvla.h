@@ -199,7 +199,7 @@ int rtvla_time_forward(rtvla_ctx* ctx, int iters, void* hip_stream, float* ms_ou
  * rtvla_linear: out[M][N] = x[M][K] w[K][N] + bias[N] (bias may be null), all bf16 row-major, fp32 accumulation,
  * K a multiple of 8, N a multiple of 16.  `tile` selects the kernel: 0 .. count-1 one block tile of the large-M MFMA
  * GEMM (rtvla_linear_tile_shape tells its rows x columns and fails past the last one), -1 the tile the forward's
- * cost model picks for this shape, RTVLA_TILE_SKINNY the weight-streaming kernel of the action expert (M <= 64,
+ * cost model picks for this shape, RTVLA_TILE_SKINNY the weight-streaming kernel of the action expert (M <= 128,
  * K = 1024, 2048 or 4096).  `nsplit`: 1 = one pass with the bias epilogue; 2..8 = split-K into fp32 partials that the
  * reduce kernel sums (N <= 2048); 0 = the split the cost model picks, through the partial + reduce route the
  * residual GEMMs of the forward take.  RTVLA_ERR_LIMIT when the tile cannot take the shape (the tiles of more than

@@ -34,10 +34,14 @@ def test_create_validates_dimensions(lib):
         with pytest.raises(capi.RtvlaError):
             capi.Context(*bad)
     with pytest.raises(capi.RtvlaError) as e:
-        capi.Context(capi.PI0, 1, 0, 64)          # 65 suffix rows do not fit the 64-row suffix tile
+        capi.Context(capi.PI0, 1, 0, 128)         # 129 suffix rows do not fit the two 64-row blocks of the action-expert kernels
+    assert e.value.code == 7
+    with pytest.raises(capi.RtvlaError) as e:
+        capi.Context(capi.DM0, 1, 10, 65)         # DM0's buffers hold one 64-row block
     assert e.value.code == 7
     capi.Context(capi.PI0, 1, 0, 63).close()
-    capi.Context(capi.PI05, 3, 52, 64).close()
+    capi.Context(capi.PI0, 1, 0, 127).close()
+    capi.Context(capi.PI05, 3, 52, 128).close()
 
 
 def test_tensor_table_matches_the_reference_layout(lib):
@@ -123,7 +127,7 @@ def test_unit_and_static_entry_points_check_sizes_before_touching_a_device(lib):
     p = ctypes.c_void_p(4096)
     assert lib.rtvla_linear_workspace_bytes(768, 1152, 3456, -1, 1) > 768 * 1152 * 2
     assert lib.rtvla_linear_workspace_bytes(16, 12, 16, -1, 1) == 0                    # K must be a multiple of 8
-    assert lib.rtvla_linear_workspace_bytes(65, 1024, 64, capi.TILE_SKINNY, 1) == 0    # the streaming kernel takes at most 64 rows
+    assert lib.rtvla_linear_workspace_bytes(129, 1024, 64, capi.TILE_SKINNY, 1) == 0   # the streaming kernel takes at most 128 rows
     assert lib.rtvla_linear(p, 16, 128, p, 16, None, p, p, 16, -1, 1, None) == capi.ERR_SIZE
     assert lib.rtvla_linear(None, 16, 128, p, 16, None, p, p, 1 << 20, -1, 1, None) == 1
     r, c = ctypes.c_int(), ctypes.c_int()
