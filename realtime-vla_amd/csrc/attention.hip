@@ -282,14 +282,11 @@ void suffix_attn_kernel(AttnP p) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
     const int nsplit = p.nsplit_eff;
-    int rowblk, split;
-    if (nsplit == 1) { rowblk = blockIdx.x; split = 0; }
-    else {                                                               // all row blocks of one split on one XCD (see mqa_kernel)
-        const int spx = (nsplit + 7) >> 3;
-        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-        split = xcd + 8 * (idx % spx); rowblk = idx / spx;
-        if (split >= nsplit) return;                                     // (whole workgroup, before any barrier)
-    }
+    // all row blocks of one split on one XCD (see mqa_kernel); the launcher uses this kernel for split passes only
+    const int spx = (nsplit + 7) >> 3;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int split = xcd + 8 * (idx % spx), rowblk = idx / spx;
+    if (split >= nsplit) return;                                         // (whole workgroup, before any barrier)
     const int m0 = rowblk * 16;
     int vl = p.prefix_alloc;
     if (p.valid_len) vl = max(0, min(*p.valid_len, p.prefix_alloc));
@@ -386,19 +383,12 @@ void suffix_attn_kernel(AttnP p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) o[i] = mfma16(vf[i][j], pb[j], o[i]);
     }
-    if (nsplit > 1) {
-        // partial record of one (row block, split): { O [DT][64] f32x4 | max [16] | sum [16] }, combined by attn_merge_kernel
-        constexpr int REC = DT * 64 * 4 + 32;
-        float* const mine = p.partial + (((size_t)batch * p.row_blocks + rowblk) * nsplit + split) * REC;
+    // partial record of one (row block, split): { O [DT][64] f32x4 | max [16] | sum [16] }, combined by attn_merge_kernel
+    constexpr int REC = DT * 64 * 4 + 32;
+    float* const mine = p.partial + (((size_t)batch * p.row_blocks + rowblk) * nsplit + split) * REC;
 #pragma unroll
-        for (int i = 0; i < DTW; ++i) *(f32x4*)(mine + ((w * DTW + i) * 64 + lane) * 4) = o[i];
-        if (w == 0 && g == 0) { mine[DT * 256 + r] = mg; mine[DT * 256 + 16 + r] = lt; }
-    } else if (row < p.rows) {
-        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-        const AttnOutRow orow = attn_out_row(p, batch, row, HD);
-#pragma unroll
-        for (int i = 0; i < DTW; ++i) store4(attn_out_at(p, orow, (w * DTW + i) * 16 + 4 * g), pack4(o[i] * inv));
-    }
+    for (int i = 0; i < DTW; ++i) *(f32x4*)(mine + ((w * DTW + i) * 64 + lane) * 4) = o[i];
+    if (w == 0 && g == 0) { mine[DT * 256 + r] = mg; mine[DT * 256 + 16 + r] = lt; }
 }
 
 // Combine the key-split partials of mqa_kernel: one wave per (row block, 16-wide d tile), 4 waves per workgroup, K/V heads
@@ -547,8 +537,8 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
     }
     p.nsplit_eff = nsplit;
     p.row_blocks = blocks;
-    if (MQ == 1 && NTK == 2 && WAVES == 4 && !CAUSAL && p.kb_per_split <= 4)          // one key block per wave: the probability-sharing kernel
-        hipLaunchKernelGGL((suffix_attn_kernel<HD>), dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(256), 0, s, p);
+    if (MQ == 1 && NTK == 2 && WAVES == 4 && !CAUSAL && nsplit > 1 && p.kb_per_split <= 4)      // one key block per wave: the probability-sharing kernel
+        hipLaunchKernelGGL((suffix_attn_kernel<HD>), dim3(8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(256), 0, s, p);
     else
     hipLaunchKernelGGL(kern, dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(WAVES * 64), smem, s, p);
     if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16, HD>), dim3(blocks * (HD / 64), p.batch), dim3(256), 0, s, p, nsplit);
