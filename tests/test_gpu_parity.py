@@ -267,6 +267,7 @@ def test_pi0_two_views_ragged_prefix():
     ("pi05", 2, 5, 64, 9),      # Pi05 with exactly one 64-row block of the action-expert kernels
     ("pi0", 1, 3, 100, 0),      # 101 suffix rows: two 64-row blocks, 51 attention row blocks
     ("pi05", 1, 5, 128, 4),     # Pi05 at the 128-row limit
+    ("pi0", 1, 2000, 20, 0),    # 2277 keys: more than four 32-key blocks per key split, i.e. the suffix pass on the general attention kernel
     ("pi05", 3, 100, 7, 0),     # Pi05, long prompt, short chunk
 ])
 def test_shape_sweep_against_the_oracle(model, views, prompt, chunk, state_tokens):
