@@ -256,9 +256,7 @@ def main():
                     help="measure the observation pre-/post-processing kernels (3 camera frames of 480x640, state, actions) instead of the forward")
     ap.add_argument("--launch-times", action="store_true",
                     help="print the mean duration of every kernel launch of one SigLIP, prefix and action-expert layer (weights cache-warm "
-                         "and cold), measured in temporary graphs, and exit.  With a tuning build of the library (build.py -DRTVLA_TUNING, "
-                         "selected by RTVLA_LIBRARY) --knockouts repeats the action-expert timings with parts of the kernels switched off")
-    ap.add_argument("--knockouts", default="", help="comma-separated RTVLA_KO masks for --launch-times (tuning builds only)")
+                         "and cold), measured in temporary graphs, and exit")
     ap.add_argument("--vendor-gemm", action="store_true",
                     help="comparator, not part of the product: time torch.matmul (the vendor GEMM library) on the GEMM shapes of the "
                          "three models, 20 launches in a graph each, and the library's own kernel for the same shape through rtvla_time_linear")
@@ -316,14 +314,6 @@ def main():
             rows.append({"layer": label, "launch": "whole layer", "warm_us": round(ctx.time_stage(stage, 3, 0, 50, stream) * 1e3, 2),
                          "cold_us": round(ctx.time_stage(stage, -1, 0, 3, stream) * 1e3, 2)})
         out = {"workload": desc, "rtvla_version": lib_version, "launches": rows}
-        if args.knockouts:
-            out["knockouts"] = []
-            for ko in args.knockouts.split(","):
-                os.environ["RTVLA_KO"] = ko
-                out["knockouts"].append({"mask": int(ko), "action_layer_launches_warm_us": {
-                    ctx.time_launch(capi.STAGE_SUFFIX_LAYER, 3, 0, idx, 100, stream)[1]: round(ctx.time_launch(capi.STAGE_SUFFIX_LAYER, 3, 0, idx, 100, stream)[0] * 1e3, 2)
-                    for idx in range(5)}})
-            os.environ["RTVLA_KO"] = "0"
         print(json.dumps(out))
         return
     if args.traffic_probe:

@@ -57,7 +57,8 @@ typedef struct rtvla_dims {
     int32_t prompt_len;      /* Pi0: rows of language_embeds; Pi05: max_prompt_len (allocated rows);
                                 DM0: max_lang_len (token ids)                                          */
     int32_t chunk_size;      /* action chunk; Pi0 suffix = chunk+1 rows, Pi05 / DM0 = chunk rows (Pi0 / Pi05: <= 128 rows, DM0: <= 64) */
-    int32_t num_steps;       /* Euler flow steps (the reference hard-codes 10; Pi05 / DM0: at most 10) */
+    int32_t num_steps;       /* Euler flow steps.  Pi0 / DM0: exactly 10, because the converted checkpoint has dt = -1/10 folded
+                                into the output projection and 10 fused time biases (RTVLA_ERR_LIMIT otherwise); Pi05: 1..10 */
     int32_t vision_layers;   /* SigLIP layers (27); DM0: ViT layers (23)                               */
     int32_t llm_layers;      /* prefix layers == action-expert layers (18; DM0: 28)                    */
 } rtvla_dims;
@@ -235,7 +236,9 @@ int rtvla_preprocess_image(const void* src_u8, int height, int width, void* dst_
  * (height x resized width x 3 bytes, resized width <= 224) exceeds that size - more than 2160 rows at full width - are
  * rejected with RTVLA_ERR_LIMIT before anything is enqueued.  All calls on one GPU share the one array: calls that
  * overlap on the same GPU (different streams or threads) race; calls on one stream are ordered.  Nothing in the array
- * has to start at zero: the horizontal pass writes every byte the vertical pass reads. */
+ * has to start at zero: the horizontal pass writes every byte the vertical pass reads.  The array's device address is
+ * looked up on the first call on each GPU; that lookup is not stream work, so the first call on a GPU must not come while
+ * `hip_stream` is being captured (RTVLA_ERR_STATE then: make one eager call first, later calls may be captured). */
 #define RTVLA_STATIC_SCRATCH_BYTES (2160 * 224 * 3)
 int rtvla_preprocess_image_static(const void* src_u8, int height, int width, void* dst_bf16, void* hip_stream);
 

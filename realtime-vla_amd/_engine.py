@@ -6,7 +6,7 @@ import os
 import torch
 
 import rtvla_capi as capi
-from tile_cache import TileCache, fingerprint
+from tile_cache import TileCache, UNTILED_WEIGHTS, fingerprint
 
 _DTYPES = {2: torch.bfloat16, 4: torch.int32}
 _ANY_ROWS = ("vision_embed_tokens_w",)          # tables whose row count is whatever the checkpoint holds
@@ -33,7 +33,7 @@ class Engine:
             vision_layers = int(checkpoint["vision_attn_qkv_w"].shape[0]) if "vision_attn_qkv_w" in checkpoint else 27
         if llm_layers is None:
             llm_layers = int(checkpoint["encoder_attn_qkv_w"].shape[0]) if "encoder_attn_qkv_w" in checkpoint else 18
-        self.model, self.vision_layers, self.llm_layers = model, vision_layers, llm_layers
+        self.model, self.vision_layers, self.llm_layers, self.num_steps = model, vision_layers, llm_layers, num_steps
         self.tile_cache = TileCache(tile_cache) if isinstance(tile_cache, (str, os.PathLike)) else tile_cache
         self.tile_cache_hit = None                                   # True / False after prepare() when a cache is in use
         self.ctx = capi.Context(model, num_views, prompt_len, chunk_size, num_steps, vision_layers, llm_layers)
@@ -65,10 +65,8 @@ class Engine:
         self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
         self.ctx.bind_workspace(self.workspace.data_ptr(), nbytes)
         # views of the library's internal activations, under the reference's buffer names where one exists
-        self.tiled_sources = {"decoder_action_fused_out_proj_w", "decoder_action_out_proj_w", "decoder_action_out_proj_b"}
         for name, off, rows, cols, ld, elem in self.ctx.buffers():
             if name.startswith("t_"):
-                self.tiled_sources.add(name[2:])                     # the weight this re-tiled copy is made from
                 continue
             flat = self.workspace[off:off + rows * ld * elem].view(torch.bfloat16 if elem == 2 else torch.float32)
             self.buffers.setdefault(name, flat.view(rows, ld)[:, :cols])
@@ -82,8 +80,11 @@ class Engine:
             torch.cuda.synchronize(self.device)
             return
         lib = capi.load()
-        ident = (lib.rtvla_tile_layout_version(), self.model, self.vision_layers, self.llm_layers)
-        key = fingerprint({k: v for k, v in self.weights.items() if k in self.tiled_sources})
+        ident = (lib.rtvla_tile_layout_version(), self.model, self.num_steps, self.vision_layers, self.llm_layers)
+        # every weight the tiled region can depend on: for Pi05 it holds W diag(1 + scale) per (flow step, layer), and scale
+        # comes from the time embeddings, the time MLP and the norm-modulation weights and biases, not only from the matrices
+        # that are re-tiled
+        key = fingerprint({k: v for k, v in self.weights.items() if k not in UNTILED_WEIGHTS})
         region = self.workspace[: self.ctx.tiled_bytes()]
         self.tile_cache_hit = self.tile_cache.load_into(key, *ident, region)
         self.ctx.prepare(self.stream.cuda_stream, tiles_loaded=self.tile_cache_hit)

@@ -523,8 +523,8 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
     auto kern = mqa_kernel<WAVES, MQ, NTK, HD, CAUSAL>;
     if (CAUSAL != (p.causal != 0)) return 1;
     if (smem > 65536) {
-        static bool done = false;
-        if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
+        static std::atomic<uint64_t> done{0};
+        if (int rc = ensure_dynamic_lds((const void*)kern, smem, done)) return rc;
     }
     const int blocks = (p.rows + 16 * MQ - 1) / (16 * MQ);
     const int nkb = (p.keys + NTK * 16 - 1) / (NTK * 16);

@@ -137,7 +137,7 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
             if (t >= HR - AIT) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                  // LDS writes of stage t+1
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (!KO(p, 2)) __syncthreads();
+        __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         // ---- second k half ----
         load_b_half(s_next, br, 0);
@@ -187,17 +187,6 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
         }
     }
     __syncthreads();                                        // the epilogue reuses the stage buffers
-    if (KO(p, 1)) {                                         // (KO 1: no epilogue; the accumulators stay live through a store that never happens)
-        float t = 0.f;
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int j = 0; j < NT; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) t += acc[i][j][e];
-        if (t == 1.2345e-30f) p.out[0] = f2bf(t);
-        return;
-    }
 
     // ---- epilogue: lane (h, r) holds rows m = m0 + 32 i + r, columns n = 32 tile + 8 grp + 4 h + e ----
     // Row-major outputs go through LDS one 32-row tile at a time so that the global stores are whole
@@ -236,8 +225,6 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
                         *(f32x4*)dst = v;
                     } else if constexpr (EPI == EPI_GEGLU) {
                         const f32x4 u = {acc[i][j + HALF][4 * grp], acc[i][j + HALF][4 * grp + 1], acc[i][j + HALF][4 * grp + 2], acc[i][j + HALF][4 * grp + 3]};
-                        if (KO(p, 4)) *(bf16x4*)dst = pack4(v[0] * u[0], v[1] * u[1], v[2] * u[2], v[3] * u[3]);      // (KO 4: no GELU)
-                        else
                         *(bf16x4*)dst = pack4(gelu_tanh(v[0]) * u[0], gelu_tanh(v[1]) * u[1], gelu_tanh(v[2]) * u[2], gelu_tanh(v[3]) * u[3]);
                     } else if constexpr (EPI == EPI_SWIGLU) {
                         const float f = p.rowscale[min(m, p.M - 1)];
@@ -274,7 +261,7 @@ RTVLA_DEVICE void gemm_block(const GemmP& p, unsigned char* smem_raw, int m0, in
                 const int row = ps * RPP + tid / CPR, ch = tid % CPR;
                 const int mm = m0 + i * 32 + row;
                 const int n = nbase + ch * (16 / ESZ);
-                if (mm < p.M && n < ncols && !KO(p, 8)) {                        // (KO 8: no global stores)
+                if (mm < p.M && n < ncols) {
                     const uint4 val = *(const uint4*)(tbuf + row * ROWB + ch * 16);
                     // (streaming hint: the output is read once by the next launch and should not displace the operand tiles in L2)
                     if constexpr (EPI == EPI_PARTIAL) __builtin_nontemporal_store(*(const f32x4*)&val, (f32x4*)(p.partial + (size_t)split * p.pstride + (size_t)mm * p.ldp + n));
@@ -443,16 +430,13 @@ int launch_cfg(const GemmP& p, hipStream_t s) {
     if ((nsplit - 1) * sps >= stages_total) return 3;      // an empty split would leave its partial unwritten
     if (MT > 4 && ((sps & 1) || (stages_total & 1))) return 3;              // the large tiles consume K stages in pairs
     GemmP q = p; q.nsplit = nsplit;
-#ifdef RTVLA_TUNING
-    q.ko = rtvla_tuning_ko();
-#endif
     // three K-stage buffers; the row-major epilogues stage 32-row output tiles in the same memory
     const size_t epi_bytes = (size_t)32 * (WN * HALF * 32 * (EPI == EPI_PARTIAL ? 4 : 2) + 16);
     const size_t smem = std::max((size_t)3 * BM * 64 * sizeof(bf16_t), epi_bytes);
     auto kern = gemm_mfma_kernel<WN, MT, NT, EPI, MIXED>;
     if (smem > 65536) {
-        static bool done = false;
-        if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
+        static std::atomic<uint64_t> done{0};
+        if (int rc = ensure_dynamic_lds((const void*)kern, smem, done)) return rc;
     }
     hipLaunchKernelGGL(kern, dim3(m_blocks * n_blocks * nsplit), dim3(WN * 64), smem, s, q, m_blocks, n_blocks, stages_total, sps, n_big);
     return hipGetLastError() == hipSuccess ? 0 : 5;

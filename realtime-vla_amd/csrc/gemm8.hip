@@ -291,8 +291,8 @@ int launch8_cfg(const GemmP& p, hipStream_t s) {
     const size_t smem = std::max((size_t)2 * MT * 32 * 64 * 2, (size_t)2 * 32 * (4 * HALF * 32 * ESZ + 16));
     auto kern = gemm8_kernel<MT, EPI, true>;
     if (smem > 65536) {
-        static bool done = false;
-        if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
+        static std::atomic<uint64_t> done{0};
+        if (int rc = ensure_dynamic_lds((const void*)kern, smem, done)) return rc;
     }
     hipLaunchKernelGGL(kern, dim3(m_blocks * n_blocks * nsplit), dim3(512), smem, s, q, m_blocks, n_blocks, stages_total, sps, n_big);
     return hipGetLastError() == hipSuccess ? 0 : 5;

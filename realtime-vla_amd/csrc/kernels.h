@@ -7,16 +7,19 @@
 #include <stdint.h>
 #include "common.h"
 
-// Tuning builds (-DRTVLA_TUNING) can knock parts of a kernel out at run time (environment variable RTVLA_KO, a bit
-// mask read at launch) to attribute its time; in the shipped build KO() is constant false and the field does not exist.
-#ifdef RTVLA_TUNING
-#define RTVLA_KO_FIELD int ko;
-#define KO(p, bit) (((p).ko & (bit)) != 0)
-int rtvla_tuning_ko();
-#else
-#define RTVLA_KO_FIELD
-#define KO(p, bit) false
-#endif
+// Kernels that need more than 64 KB of dynamic LDS have the limit raised once per device: the attribute belongs to the
+// device's copy of the kernel, so a process that drives several GPUs sets it on each.  `done` is one bit mask per kernel
+// instantiation (a function-local static of its launcher).  Returns 0 or the launcher error code 4.
+#include <atomic>
+inline int ensure_dynamic_lds(const void* kernel, size_t bytes, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 4;
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && (done.load(std::memory_order_acquire) >> dev & 1)) return 0;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return 4;
+    if (tracked) done.fetch_or((uint64_t)1 << dev, std::memory_order_release);
+    return 0;
+}
 
 // ----- pre-tiled weights ------------------------------------------------------------
 // A weight W[K][N] (row-major, "in x out") is re-laid out once as MFMA operand fragments:
@@ -67,7 +70,6 @@ struct GemmP {
     float* partial; int ldp; size_t pstride;   // [split][row][ldp]
     const bf16_t* rope;                        // [row][256] = cos0 sin0 cos1 sin1 ...
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt;
-    RTVLA_KO_FIELD
 };
 // workgroup tile (rows x columns), 4 waves each owning 64 columns (two 32-column MFMA tiles).  The tiles of 128 rows and
 // more by 256 columns are upper bounds: their launches mix row blocks of that many and of 32 fewer rows so that the
@@ -119,7 +121,6 @@ struct SkinnyP {
                                                // (Pi05: the shift of the adaptive RMS norm times the weights, see Sched::prepare)
     const bf16_t* rope;                        // [row][256]
     bf16_t* q; bf16_t* k; bf16_t* vt; int ldvt; int kv_row0;
-    RTVLA_KO_FIELD
 };
 int launch_skinny(const SkinnyP& p, int epi, hipStream_t s);
 
@@ -153,7 +154,6 @@ struct AttnP {
     // key split over workgroups (nsplit > 1, at most 16): fp32 partial records, combined by a second launch
     int nsplit; float* partial; size_t partial_floats;
     int kb_per_split, nsplit_eff, row_blocks;    // filled by the launcher
-    RTVLA_KO_FIELD
 };
 // Gemma (HD 256): many rows, two row tiles per workgroup / few rows, one row tile and a key split; DM0 grouped-query (HD 128)
 // prefix and suffix (the ViT attention, HD 64, is launch_flash_attention)

@@ -4,6 +4,7 @@
 // touch only caller-owned memory, so the whole forward can be captured into one HIP graph.
 #include "../../include/rtvla.h"
 #include "kernels.h"
+#include "tuning.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -11,10 +12,6 @@
 #include <map>
 #include <string>
 #include <vector>
-
-#ifdef RTVLA_TUNING
-int rtvla_tuning_ko() { const char* e = getenv("RTVLA_KO"); return e ? atoi(e) : 0; }
-#endif
 
 namespace {
 
@@ -91,8 +88,6 @@ struct rtvla_ctx {
     }
     bf16_t* TW(const char* n, int layer = 0) { const WsBuf& b = BI(n); return (bf16_t*)(ws + b.offset) + (size_t)b.ld * layer; }
 
-    int attn_split = 0;            // suffix attention key split; 0: one workgroup per 128 keys
-
     int only = -1;                 // >= 0: enqueue only the launch with this index (per-kernel timing)
     std::string last_name;
     bool want(const char* what) {
@@ -124,15 +119,7 @@ constexpr int64_t ATTN_PARTIAL_FLOATS = 64 * 16 * (16 * 64 * 4 + 32);   // 64 ro
 TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittable, const char* what, int eight = 0) {
     static const int tiles[] = {TILE_224x256, TILE_192x256, TILE_160x256, TILE_128x256, TILE_64x256, TILE_128x128, TILE_64x128};
     static const int splits[] = {1, 2, 3, 4, 6, 8};
-#ifdef RTVLA_TUNING
-    // tuning builds only: force tile / split for the launches whose name contains RTVLA_FORCE_FOR
-    const char* only_for = getenv("RTVLA_FORCE_FOR");
-    if (const char* e = (only_for && !strstr(what, only_for)) ? nullptr : getenv("RTVLA_FORCE_TILE")) {
-        TileChoice c{atoi(e), 1};
-        if (const char* s = getenv("RTVLA_FORCE_SPLIT")) if (splittable) c.nsplit = atoi(s);
-        return c;
-    }
-#endif
+    { TileChoice forced; if (tuning_forced_tile(what, splittable, &forced.tile, &forced.nsplit)) return forced; }
     // measured (M = 8115, K = 1024, N = 4096, bias + GELU): the eight-wave 256 x 256 tile takes 84-89 us where the best four-wave
     // tile takes 98-101 us; with 788 rows, with the gated epilogues and with fp32 split-K partials the four-wave tiles win
     // (eight: 1 = bias (+ GELU) epilogue, 2 = the ViT QKV epilogue, measured 75 us with the eight-wave 128 x 256 tile against 93 us)
@@ -180,10 +167,7 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
             if (t < best) { best = t; bc = TileChoice{tile, sp}; }
         }
     }
-#ifdef RTVLA_TUNING
-    if (getenv("RTVLA_PRINT_TILES")) fprintf(stderr, "rtvla tile choice: %-18s M=%d N=%d stages=%d -> %dx%d split %d (model %.1f us)\n", what, M, ncols16 * 16,
-                                             stages, gemm_tile_bm(bc.tile), gemm_tile_bn(bc.tile), bc.nsplit, best);
-#endif
+    tuning_report_tile(what, M, ncols16 * 16, stages, gemm_tile_bm(bc.tile), gemm_tile_bn(bc.tile), bc.nsplit, best);
     return bc;
 }
 
@@ -614,7 +598,7 @@ struct Sched {
         a.q = c->B("decoder_q_buf"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
         a.out = c->B("decoder_attn"); a.group = 8; a.out_tiled = 1; a.out_cols32 = 64; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
-        a.nsplit = c->attn_split > 0 ? c->attn_split : std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
+        a.nsplit = std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
         if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_SUFFIX, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
         skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
@@ -681,8 +665,10 @@ struct Sched {
         GemmP u{}; u.out = c->B("vision_fc"); u.ldo = 4096; u.bias_f32 = WF("vision_fused_fc_b", 4096, i);
         gemm(c->B("vision_x_norm"), 1024, M, M, c->TW("t_vision_fused_fc_w", i), nullptr, 1024, 4096, EPI_BIAS_GELU, u, "vit fc");
         gemm(c->B("vision_fc"), 4096, M, M, c->TW("t_vision_proj_w", i), nullptr, 4096, 1024, EPI_PARTIAL, GemmP{}, "vit proj");
-        reduce(M, 1024, c->W("vision_proj_b", 1024, i), c->B("vision_x_2d"), 1024, c->B("vision_x_2d"), 1024, c->B("vision_x_norm"), 1024,
-               NORM_LAYER, c->B("const_ones"), c->B("const_zeros"), 1e-5f, last_split, "vit proj reduce");
+        // (nothing reads the normalised copy after the last layer: the down-sampling convolutions take the stream itself)
+        const bool last = i == d.vision_layers - 1;
+        reduce(M, 1024, c->W("vision_proj_b", 1024, i), c->B("vision_x_2d"), 1024, c->B("vision_x_2d"), 1024, last ? nullptr : c->B("vision_x_norm"), 1024,
+               last ? NORM_NONE : NORM_LAYER, c->B("const_ones"), c->B("const_zeros"), 1e-5f, last_split, "vit proj reduce");
     }
 
     // dm0_infer.py:738-756: drop the class token, two stride-2 3x3 convolutions, projector, token embeddings; then the RMS
@@ -716,6 +702,7 @@ struct Sched {
                                    c->W("prefix_rope_weights"), c->B("prefix_Q"), qstride, dK(i), (size_t)kp * 128, dVt(i), (size_t)128 * kp, kp >> 5, 0, P, s);
             c->note(0, "prefix qk-norm rope");
         }
+        if (i == d.llm_layers - 1) return;           // the action expert reads only the K / V cache of the last prefix layer
         AttnP a{};
         a.q = c->B("prefix_Q"); a.k = dK(i); a.vt = dVt(i); a.ldvt = kp;
         a.batch = 8; a.q_bstride = qstride; a.k_bstride = (size_t)kp * 128; a.vt_bstride = (size_t)128 * kp;
@@ -759,7 +746,7 @@ struct Sched {
         a.batch = 8; a.q_bstride = (size_t)128 * 128; a.k_bstride = (size_t)kp * 128; a.vt_bstride = (size_t)128 * kp;
         a.group = 2; a.rows = 2 * ch; a.keys = P + ch; a.scale = 0.08838834764831845f; a.prefix_alloc = P + ch;
         a.out = c->B("decoder_attn"); a.out_tiled = 1; a.out_bcol = 256; a.out_cols32 = 64;
-        a.nsplit = c->attn_split > 0 ? c->attn_split : std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
+        a.nsplit = std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
         if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_GQA128_SUFFIX, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024;
         skinny(c->B("decoder_attn"), 2048, ch, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
@@ -981,7 +968,9 @@ int rtvla_create(const rtvla_dims* dims, rtvla_ctx** out) {
     if (d.vision_layers < 1 || d.llm_layers < 1) return RTVLA_ERR_ARG;
     const int S_d = d.chunk_size + (d.model == RTVLA_PI0 ? 1 : 0);
     if (S_d > (d.model == RTVLA_DM0 ? 64 : 128)) return RTVLA_ERR_LIMIT;        // two 64-row blocks of the action-expert kernels (DM0's buffers hold one)
-    if (d.model != RTVLA_PI0 && d.num_steps > 10) return RTVLA_ERR_LIMIT;       // the per-step time tables have 10 rows
+    // Pi0 / DM0: the converted checkpoint is tied to 10 steps (dt = -1/10 folded into the output projection, 10 fused time
+    // biases: convert_from_jax.py:176-194); Pi05 scales by -1/num_steps itself but its time table has 10 rows
+    if (d.model == RTVLA_PI05 ? d.num_steps > 10 : d.num_steps != 10) return RTVLA_ERR_LIMIT;
     if (d.prompt_len > 4096) return RTVLA_ERR_LIMIT;
     rtvla_ctx* c = new (std::nothrow) rtvla_ctx();
     if (!c) return RTVLA_ERR_ARG;

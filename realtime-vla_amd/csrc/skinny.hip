@@ -39,13 +39,13 @@ void skinny_kernel(SkinnyP p) {
     // ---- weight fragments: the HBM stream, all in flight at once ----
     bf16x8 b[NB][KBW];
     {
-        const bf16_t* bp0 = p.B0 + ((size_t)(KO(p, 1) ? 0 : tile) * p.K32p + kb0) * 512 + lane * 8;       // (KO 1: every workgroup reads tile 0 -> cache hits)
+        const bf16_t* bp0 = p.B0 + ((size_t)tile * p.K32p + kb0) * 512 + lane * 8;
 #pragma unroll
-        for (int i = 0; i < KBW; ++i) b[0][i] = *(const bf16x8*)(bp0 + (size_t)(KO(p, 2) ? 0 : i) * 512);
+        for (int i = 0; i < KBW; ++i) b[0][i] = *(const bf16x8*)(bp0 + (size_t)i * 512);
         if constexpr (DUAL) {
-            const bf16_t* bp1 = p.B1 + ((size_t)(KO(p, 1) ? 0 : tile) * p.K32p + kb0) * 512 + lane * 8;
+            const bf16_t* bp1 = p.B1 + ((size_t)tile * p.K32p + kb0) * 512 + lane * 8;
 #pragma unroll
-            for (int i = 0; i < KBW; ++i) b[1][i] = *(const bf16x8*)(bp1 + (size_t)(KO(p, 2) ? 0 : i) * 512);
+            for (int i = 0; i < KBW; ++i) b[1][i] = *(const bf16x8*)(bp1 + (size_t)i * 512);
         }
     }
     // activation fragments: with the fragment-tiled layout (and no row offset) each is one
@@ -154,14 +154,12 @@ void skinny_kernel(SkinnyP p) {
     }
 
     // ---- reduce the 8 K-slices through LDS; wave mt finishes row tile mt ----
-    if (KO(p, 16)) return;                                   // (KO 16: loads and MFMAs only)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mt = 0; mt < SK_MTS; ++mt) red[((size_t)w * NB * SK_MTS + nb * SK_MTS + mt) * 64 + lane] = acc[nb][mt];
     __syncthreads();
     if (w >= SK_MTS) return;
-    if (KO(p, 32)) return;                                   // (KO 32: no cross-wave sum, no epilogue)
     const int mt = w;
     const int m = m_base + mt * 16 + r;
     f32x4 v[NB];
@@ -231,16 +229,10 @@ int launch_inst(const SkinnyP& p, hipStream_t s) {
     const size_t smem = (size_t)SK_WAVES * NB * SK_MTS * 64 * 16 + (size_t)SK_WAVES * 64 * 4;
     auto kern = skinny_kernel<NCH, NORM, EPI, SK_MTS>;
     if (smem > 65536) {
-        static bool done = false;
-        if (!done) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return 4; done = true; }
+        static std::atomic<uint64_t> done{0};
+        if (int rc = ensure_dynamic_lds((const void*)kern, smem, done)) return rc;
     }
-#ifdef RTVLA_TUNING
-    SkinnyP q = p; q.ko = rtvla_tuning_ko();
-    if (q.ko & 4) { hipLaunchKernelGGL(kern, dim3(1, 1), dim3(SK_WAVES * 64), smem, s, q); return 0; }      // KO 4: one workgroup (launch floor)
-    hipLaunchKernelGGL(kern, dim3(p.N16, (p.M + SK_MTS * 16 - 1) / (SK_MTS * 16)), dim3(SK_WAVES * 64), smem, s, q);
-#else
     hipLaunchKernelGGL(kern, dim3(p.N16, (p.M + SK_MTS * 16 - 1) / (SK_MTS * 16)), dim3(SK_WAVES * 64), smem, s, p);
-#endif
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 

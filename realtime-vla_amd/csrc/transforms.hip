@@ -153,8 +153,8 @@ int preprocess_image_impl(const void* src_u8, int height, int width, void* dst_b
     if ((int)ceil(sx > 1.0 ? sx : 1.0) * 2 + 1 > MAX_TAPS || (int)ceil(sy > 1.0 ? sy : 1.0) * 2 + 1 > MAX_TAPS) return RTVLA_ERR_LIMIT;
     if (scratch_bytes < (size_t)height * rw * 3) return too_small_code;
     uint8_t* tmp = nullptr;
-    if (int rc = get_scratch(&tmp)) return rc;
     hipStream_t s = (hipStream_t)stream;
+    if (int rc = get_scratch(&tmp, s)) return rc;
     const int n1 = height * rw;
     hipLaunchKernelGGL(resample_h_kernel, dim3((n1 + 255) / 256), dim3(256), 0, s, (const uint8_t*)src_u8, height, width, rw, tmp);
     hipLaunchKernelGGL(resample_v_pad_norm_kernel, dim3((224 * 224 + 255) / 256), dim3(256), 0, s, (const uint8_t*)tmp, height, rw, rh,
@@ -167,11 +167,16 @@ constexpr int MAX_DEVICES = 64;
 std::mutex static_scratch_mutex;
 void* static_scratch_addr[MAX_DEVICES] = {};
 
-int static_scratch_ptr(uint8_t** out) {
+// The lookup loads the code object and is not stream work: it must not happen while `s` is being captured into a graph,
+// so a first call on a device that comes under capture is refused (RTVLA_ERR_STATE) and any earlier eager call resolves it.
+int static_scratch_ptr(uint8_t** out, hipStream_t s) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return RTVLA_ERR_DEVICE;
     std::lock_guard<std::mutex> lock(static_scratch_mutex);
     if (!static_scratch_addr[dev]) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cap) != hipSuccess) return RTVLA_ERR_DEVICE;
+        if (cap != hipStreamCaptureStatusNone) return RTVLA_ERR_STATE;
         void* ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return RTVLA_ERR_DEVICE;
         static_scratch_addr[dev] = ptr;
@@ -192,7 +197,7 @@ size_t rtvla_preprocess_image_scratch(int height, int width) {
 int rtvla_preprocess_image(const void* src_u8, int height, int width, void* dst_bf16, void* scratch_arg, size_t scratch_bytes, void* stream) {
     if (!scratch_arg) return RTVLA_ERR_ARG;
     return preprocess_image_impl(src_u8, height, width, dst_bf16, scratch_bytes, RTVLA_ERR_SIZE,
-                                 [&](uint8_t** out) { *out = (uint8_t*)scratch_arg; return (int)RTVLA_OK; }, stream);
+                                 [&](uint8_t** out, hipStream_t) { *out = (uint8_t*)scratch_arg; return (int)RTVLA_OK; }, stream);
 }
 
 int rtvla_preprocess_image_static(const void* src_u8, int height, int width, void* dst_bf16, void* stream) {

@@ -7,7 +7,7 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.environ.get("RTVLA_LIBRARY") or os.path.join(HERE, "librtvla.so")   # override: an alternative build of the same ABI
+LIB_PATH = os.path.join(HERE, "librtvla.so")
 
 PI0, PI05, DM0 = 0, 1, 2
 

@@ -1,13 +1,16 @@
 """On-disk cache of the library's re-tiled weights.
 
-The first rtvla_tiled_bytes bytes of the workspace after rtvla_prepare are a pure function of the checkpoint, the
-model kind, the layer counts and the tile layout version.  This module saves that region once per checkpoint and,
-on later starts, memory-maps the file and copies it to the device instead of re-tiling.  The file is keyed by a
+The first rtvla_tiled_bytes bytes of the workspace after rtvla_prepare are a function of the checkpoint's weights, the
+model kind, the layer counts, the number of flow steps and the tile layout version.  For Pi0 and DM0 only the re-tiled
+matrices enter; for Pi05 the region also holds W diag(1 + scale) per (flow step, layer), and `scale` comes from the time
+embedding table, the time MLP and the norm-modulation weights and biases, so the key has to cover every weight of the
+checkpoint except the ones that are never tiled (token-embedding tables, prompt embeddings).  This module saves that
+region once per checkpoint and, on later starts, memory-maps the file and copies it to the device instead of re-tiling.  The file is keyed by a
 fingerprint of the weights computed on the device where they already are (exact integer sums, so it is
 deterministic and costs one pass over the weights at memory bandwidth), not by a path or a time stamp.
 
     file = <dir>/<key>.rtvla-tiles :  64-byte little-endian header | the tiled region, byte for byte
-    header: b"RTVLATIL" | u32 layout version | u32 model | u32 vision layers | u32 llm layers | u64 tiled bytes | 32-byte key
+    header: b"RTVLATIL" | u32 layout version | u16 model | u16 flow steps | u32 vision layers | u32 llm layers | u64 tiled bytes | 32-byte key
 """
 import hashlib
 import os
@@ -16,8 +19,10 @@ import struct
 import torch
 
 MAGIC = b"RTVLATIL"
-HEADER = struct.Struct("<8sIIIIQ32s")
+HEADER = struct.Struct("<8sIHHIIQ32s")
 assert HEADER.size == 64
+# weights that never reach the tiled region: the prompt's embeddings and the token-embedding tables (about 1 GB each)
+UNTILED_WEIGHTS = ("language_embeds", "embedding_weight", "vision_embed_tokens_w")
 
 
 def fingerprint(weights):
@@ -46,7 +51,7 @@ class TileCache:
     def path(self, key):
         return os.path.join(self.directory, key.hex()[:40] + ".rtvla-tiles")
 
-    def load_into(self, key, layout_version, model, vision_layers, llm_layers, region):
+    def load_into(self, key, layout_version, model, num_steps, vision_layers, llm_layers, region):
         """Copy the cached region into `region` (a uint8 device tensor of exactly the tiled size).  False when there is
         no file for this key or its header does not match in every field."""
         path = self.path(key)
@@ -55,22 +60,22 @@ class TileCache:
             if os.path.getsize(path) != HEADER.size + n:
                 return False
             with open(path, "rb") as f:
-                magic, ver, mdl, vl, ll, size, k = HEADER.unpack(f.read(HEADER.size))
+                magic, ver, mdl, steps, vl, ll, size, k = HEADER.unpack(f.read(HEADER.size))
         except (OSError, struct.error):
             return False
-        if (magic, ver, mdl, vl, ll, size, k) != (MAGIC, layout_version, model, vision_layers, llm_layers, n, key):
+        if (magic, ver, mdl, steps, vl, ll, size, k) != (MAGIC, layout_version, model, num_steps, vision_layers, llm_layers, n, key):
             return False
         mapped = torch.from_file(path, shared=False, size=HEADER.size + n, dtype=torch.uint8)     # memory-mapped, read as it is copied
         region.copy_(mapped[HEADER.size:])
         return True
 
-    def store(self, key, layout_version, model, vision_layers, llm_layers, region):
+    def store(self, key, layout_version, model, num_steps, vision_layers, llm_layers, region):
         os.makedirs(self.directory, exist_ok=True)
         path = self.path(key)
         tmp = path + ".tmp.%d" % os.getpid()
         host = region.cpu()
         with open(tmp, "wb") as f:
-            f.write(HEADER.pack(MAGIC, layout_version, model, vision_layers, llm_layers, host.numel(), key))
+            f.write(HEADER.pack(MAGIC, layout_version, model, num_steps, vision_layers, llm_layers, host.numel(), key))
             f.write(host.numpy().tobytes() if host.numel() < (1 << 28) else b"")
             if host.numel() >= (1 << 28):                      # large regions in pieces, without a second host copy
                 step = 1 << 28

@@ -39,6 +39,13 @@ def test_create_validates_dimensions(lib):
     with pytest.raises(capi.RtvlaError) as e:
         capi.Context(capi.DM0, 1, 10, 65)         # DM0's buffers hold one 64-row block
     assert e.value.code == 7
+    # the converted Pi0 / DM0 checkpoints are tied to 10 flow steps (dt folded into the output projection, 10 time biases);
+    # Pi05 scales by -1/num_steps itself and takes 1..10
+    for model, steps in ((capi.PI0, 5), (capi.PI0, 11), (capi.PI0, 20), (capi.DM0, 9), (capi.PI05, 11)):
+        with pytest.raises(capi.RtvlaError) as e:
+            capi.Context(model, 1, 4, 10, steps)
+        assert e.value.code == 7, (model, steps)
+    capi.Context(capi.PI05, 1, 4, 10, 4).close()
     capi.Context(capi.PI0, 1, 0, 63).close()
     capi.Context(capi.PI0, 1, 0, 127).close()
     capi.Context(capi.PI05, 3, 52, 128).close()

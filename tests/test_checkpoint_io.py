@@ -76,15 +76,15 @@ def test_tile_cache_file_round_trip_and_header_checks(tmp_path):
     cache = tc.TileCache(tmp_path / "tiles")
     key = bytes(range(32))
     region = torch.arange(5000, dtype=torch.int64).to(torch.uint8)
-    assert not cache.load_into(key, 2, 0, 27, 18, torch.empty_like(region))               # nothing stored yet
-    path = cache.store(key, 2, 0, 27, 18, region)
+    assert not cache.load_into(key, 2, 0, 10, 27, 18, torch.empty_like(region))               # nothing stored yet
+    path = cache.store(key, 2, 0, 10, 27, 18, region)
     assert os.path.getsize(path) == 64 + 5000
     back = torch.zeros_like(region)
-    assert cache.load_into(key, 2, 0, 27, 18, back) and torch.equal(back, region)
-    for other in ((3, 0, 27, 18), (2, 1, 27, 18), (2, 0, 2, 18), (2, 0, 27, 2)):           # layout version, model, layer counts
+    assert cache.load_into(key, 2, 0, 10, 27, 18, back) and torch.equal(back, region)
+    for other in ((3, 0, 10, 27, 18), (2, 1, 10, 27, 18), (2, 0, 5, 27, 18), (2, 0, 10, 2, 18), (2, 0, 10, 27, 2)):   # layout version, model, flow steps, layer counts
         assert not cache.load_into(key, *other, torch.zeros_like(region))
-    assert not cache.load_into(key, 2, 0, 27, 18, torch.zeros(4999, dtype=torch.uint8))  # another size
-    assert not cache.load_into(bytes(32), 2, 0, 27, 18, torch.zeros_like(region))         # another checkpoint
+    assert not cache.load_into(key, 2, 0, 10, 27, 18, torch.zeros(4999, dtype=torch.uint8))  # another size
+    assert not cache.load_into(bytes(32), 2, 0, 10, 27, 18, torch.zeros_like(region))         # another checkpoint
     with open(path, "r+b") as f:                                                           # a truncated / foreign file
         f.write(b"garbage!")
-    assert not cache.load_into(key, 2, 0, 27, 18, torch.zeros_like(region))
+    assert not cache.load_into(key, 2, 0, 10, 27, 18, torch.zeros_like(region))

@@ -458,3 +458,12 @@ def test_start_from_the_tile_cache_gives_bit_identical_actions(tmp_path):
     b = Pi05Inference(ck5, 1, 6, discrete_state_input=False, tile_cache=tmp_path)
     assert (a._engine.tile_cache_hit, b._engine.tile_cache_hit) == (False, True)
     assert torch.equal(a.forward(img5, noise5), b.forward(img5, noise5))
+    # the cached region holds W diag(1 + scale) per (flow step, layer): a checkpoint that differs only in a tensor the scale
+    # is computed from (here a norm-modulation bias, which is not itself re-tiled) must miss the cache
+    ck6 = dict(ck5); ck6["decoder_pre_attn_norm_mod_b"] = ck5["decoder_pre_attn_norm_mod_b"].clone()
+    ck6["decoder_pre_attn_norm_mod_b"][0, :1024] += 0.25
+    files = len(list(tmp_path.iterdir()))
+    c = Pi05Inference(ck6, 1, 6, discrete_state_input=False, tile_cache=tmp_path)
+    assert c._engine.tile_cache_hit is False and len(list(tmp_path.iterdir())) == files + 1
+    uncached = Pi05Inference(ck6, 1, 6, discrete_state_input=False).forward(img5, noise5).clone()
+    assert torch.equal(c.forward(img5, noise5), uncached) and not torch.equal(uncached, a.forward(img5, noise5))

@@ -50,3 +50,28 @@ def test_static_scratch_entry_point_equals_the_workspace_one_on_consecutive_call
     assert torch.equal(x, y)
     with pytest.raises(ValueError):
         tr.resize_pad_normalize_into(tall, out, static_scratch=True)
+
+
+def test_static_scratch_entry_point_inside_a_captured_graph():
+    """The advertised use: the call recorded into a HIP graph (nothing may allocate there) and replayed on other frames."""
+    import rtvla_capi as capi
+    lib = capi.load()
+    h, w = 480, 640
+    frames = [_frame(20 + i, h, w) for i in range(3)]
+    src = frames[0].clone()
+    out = torch.zeros(224, 224, 3, dtype=torch.bfloat16, device="cuda:0")
+    # one eager call first: it resolves the static array's address on this GPU, which a captured call may not do
+    assert lib.rtvla_preprocess_image_static(_P(src.data_ptr()), h, w, _P(out.data_ptr()), _P(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.rtvla_preprocess_image_static(_P(src.data_ptr()), h, w, _P(out.data_ptr()), _P(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    for f in frames[1:] + frames[:1]:
+        src.copy_(f)
+        out.fill_(7.0)
+        torch.cuda.synchronize()                       # eager work and a synchronisation between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        want, _ = _both(lib, f)
+        assert torch.equal(out.cpu(), want)
