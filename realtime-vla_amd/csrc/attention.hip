@@ -19,8 +19,12 @@
 // L2 port, so a workgroup that walks all keys is bound by that port.  Its keys are therefore split over
 // several workgroups, each writing an un-normalised partial (O, row max, row sum); a second small
 // kernel (attn_merge_kernel) combines the partials.  Merging inside the first kernel (last workgroup to
-// finish does it) was measured slower: the partials cross XCDs, whose L2s are not coherent with each
-// other, and device-scope fences or write-through accesses cost more than one extra launch.
+// finish does it) was measured slower, twice: with the partials crossing XCDs, whose L2s are not coherent with each
+// other, device-scope fences or write-through accesses cost more than one extra launch; and with all key splits of a
+// row block dealt to ONE XCD (no fence at all: write-through stores, an arrival counter in that XCD's L2, the last
+// workgroup reading the others' records from the cache they were written to) the single launch took 8.3 us against 7.7 us
+// for the pair - store acknowledge, atomic round trip and the dependent loads of the tail add up to a launch boundary,
+// and every XCD then fetches all of K / V^T.
 #include "kernels.h"
 
 namespace {
@@ -281,10 +285,16 @@ void suffix_attn_kernel(AttnP p) {
     const bf16_t* const vbase = p.vt + (size_t)batch * p.vt_bstride;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int g = lane >> 4, r = lane & 15;
+    const int riders = p.riders;                                         // a multiple of 8, so that the decode below still sees the XCD in the low bits
+    if ((int)blockIdx.x < riders) {                                      // riding workgroups: weight tiles of a later launch
+        if (blockIdx.y == 0) prefetch_tile<256>(p.pf_attn, blockIdx.x, tid);
+        return;
+    }
     const int nsplit = p.nsplit_eff;
     // all row blocks of one split on one XCD (see mqa_kernel); the launcher uses this kernel for split passes only
     const int spx = (nsplit + 7) >> 3;
-    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int bx = blockIdx.x - riders;
+    const int xcd = bx & 7, idx = bx >> 3;
     const int split = xcd + 8 * (idx % spx), rowblk = idx / spx;
     if (split >= nsplit) return;                                         // (whole workgroup, before any barrier)
     const int m0 = rowblk * 16;
@@ -518,7 +528,7 @@ void vision_attn_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 }
 
 template <int WAVES, int MQ, int NTK, int HD, bool CAUSAL = false>
-int launch_mqa_inst(AttnP p, hipStream_t s) {
+int launch_mqa_inst(AttnP p, hipStream_t s, int* nk) {
     const size_t smem = (size_t)WAVES * (HD / 16) * 64 * 16 + (size_t)2 * WAVES * MQ * 16 * 4;
     auto kern = mqa_kernel<WAVES, MQ, NTK, HD, CAUSAL>;
     if (CAUSAL != (p.causal != 0)) return 1;
@@ -537,28 +547,31 @@ int launch_mqa_inst(AttnP p, hipStream_t s) {
     }
     p.nsplit_eff = nsplit;
     p.row_blocks = blocks;
-    if (MQ == 1 && NTK == 2 && WAVES == 4 && !CAUSAL && nsplit > 1 && p.kb_per_split <= 4)      // one key block per wave: the probability-sharing kernel
-        hipLaunchKernelGGL((suffix_attn_kernel<HD>), dim3(8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(256), 0, s, p);
-    else
+    if (MQ == 1 && NTK == 2 && WAVES == 4 && !CAUSAL && nsplit > 1 && p.kb_per_split <= 4) {    // one key block per wave: the probability-sharing kernel
+        p.riders = prefetch_wgs(p.pf_attn);
+        if (p.riders & 7) return 1;
+        hipLaunchKernelGGL((suffix_attn_kernel<HD>), dim3(8 * ((nsplit + 7) / 8) * blocks + p.riders, p.batch), dim3(256), 0, s, p);
+    } else
     hipLaunchKernelGGL(kern, dim3(nsplit == 1 ? blocks : 8 * ((nsplit + 7) / 8) * blocks, p.batch), dim3(WAVES * 64), smem, s, p);
     if (nsplit > 8) hipLaunchKernelGGL((attn_merge_kernel<MQ, 16, HD>), dim3(blocks * (HD / 64), p.batch), dim3(256), 0, s, p, nsplit);
     else if (nsplit > 1) hipLaunchKernelGGL((attn_merge_kernel<MQ, 8, HD>), dim3(blocks * (HD / 64), p.batch), dim3(256), 0, s, p, nsplit);
+    if (nk) *nk = nsplit > 1 ? 2 : 1;
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 
 }  // namespace
 
-int launch_mqa_attention(const AttnP& p0, int variant, hipStream_t s) {
+int launch_mqa_attention(const AttnP& p0, int variant, hipStream_t s, int* nk) {
     AttnP p = p0;
     if (p.rows <= 0 || p.keys <= 0 || (p.ldvt & 31) || p.ldvt < ((p.keys + 31) / 32) * 32) return 1;
     if (p.batch < 1) p.batch = 1;
     if (p.batch_inner < 1) p.batch_inner = 1;
     if (p.group < 1) return 1;
     switch (variant) {                                          // template: waves, row tiles per workgroup, 16-key tiles per wave round, head width
-        case ATTN_PREFIX: return launch_mqa_inst<4, 2, 2, 256>(p, s);
-        case ATTN_SUFFIX: return launch_mqa_inst<4, 1, 2, 256>(p, s);
-        case ATTN_GQA128_PREFIX: return launch_mqa_inst<4, 2, 2, 128, true>(p, s);
-        case ATTN_GQA128_SUFFIX: return launch_mqa_inst<4, 1, 2, 128>(p, s);
+        case ATTN_PREFIX: return launch_mqa_inst<4, 2, 2, 256>(p, s, nk);
+        case ATTN_SUFFIX: return launch_mqa_inst<4, 1, 2, 256>(p, s, nk);
+        case ATTN_GQA128_PREFIX: return launch_mqa_inst<4, 2, 2, 128, true>(p, s, nk);
+        case ATTN_GQA128_SUFFIX: return launch_mqa_inst<4, 1, 2, 128>(p, s, nk);
     }
     return 2;
 }

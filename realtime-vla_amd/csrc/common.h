@@ -100,3 +100,39 @@ RTVLA_DEVICE float wave_sum(float v) {
     for (int o = 8; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
 }
+
+// Pulling weight tiles that a LATER launch of the same graph will stream towards the caches: every thread reads one word of
+// each 128-byte line of its share of a tile and throws it away (the empty asm keeps the loads alive and makes the wave wait for
+// them before it ends).  The lines land in the memory-side cache and in the L2 of the XCD the workgroup runs on, so the
+// callers give workgroup e the tile that the consuming launch will process on the same XCD (tile index = workgroup index
+// modulo 8 when both grids are dealt round-robin over the XCDs).  A launch cannot end before its riders' loads have come
+// back, and such touches draw only ~3.5 TB/s from HBM: measured on the action expert, riders that fetch the 4 MB of the
+// output projection during the suffix attention pay (0.7 us per layer), riders that fetch the 16.8 MB of the gate / up weights
+// during the attention or the merge launch lengthen that launch by 4-6 us and save 2.3 us in the consumer.
+struct PrefetchP {
+    const char* base[4];        // up to four weight blocks
+    int tile_bytes[4];          // contiguous bytes per tile (at most 4 x 128 x the workgroup's thread count)
+    int n_tiles[4];             // tiles (= riding workgroups) per block, multiples of 8; 0 ends the list
+};
+static inline int prefetch_wgs(const PrefetchP& p) { int n = 0; for (int k = 0; k < 4 && p.n_tiles[k] > 0; ++k) n += p.n_tiles[k]; return n; }
+template <int NTHREADS>
+RTVLA_DEVICE void prefetch_tile(const PrefetchP& p, int e, int tid) {
+    // every field is read before the first branch: one round of scalar loads instead of a dependent chain
+    const int n0 = p.n_tiles[0], n1 = p.n_tiles[1], n2 = p.n_tiles[2], n3 = p.n_tiles[3];
+    const int b0 = p.tile_bytes[0], b1 = p.tile_bytes[1], b2 = p.tile_bytes[2], b3 = p.tile_bytes[3];
+    const char* const a0 = p.base[0]; const char* const a1 = p.base[1]; const char* const a2 = p.base[2]; const char* const a3 = p.base[3];
+    const int e1 = e - n0, e2 = e1 - n1, e3 = e2 - n2;
+    const char* a = a0; int bytes = b0, idx = e;
+    if (e1 >= 0) { a = a1; bytes = b1; idx = e1; }
+    if (e2 >= 0) { a = a2; bytes = b2; idx = e2; }
+    if (e3 >= 0) { a = a3; bytes = b3; idx = e3; }
+    if (e3 >= n3) return;
+    const char* t = a + (size_t)idx * bytes;
+    unsigned v[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int off = min((i * NTHREADS + tid) * 128, bytes - 128);       // (tiles shorter than the unrolled reach re-read their last line)
+        v[i] = *(const unsigned*)(t + off);
+    }
+    asm volatile("" ::"v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]));
+}

@@ -154,11 +154,15 @@ struct AttnP {
     // key split over workgroups (nsplit > 1, at most 16): fp32 partial records, combined by a second launch
     int nsplit; float* partial; size_t partial_floats;
     int kb_per_split, nsplit_eff, row_blocks;    // filled by the launcher
+    // key-split suffix passes only: weight tiles of a later launch that extra ("riding") workgroups of the attention launch pull
+    // towards the caches (the launch streams no weights itself and its grid leaves CUs idle)
+    PrefetchP pf_attn;
+    int riders;                                  // filled by the launcher: riding workgroups, first in the grid (a multiple of 8)
 };
 // Gemma (HD 256): many rows, two row tiles per workgroup / few rows, one row tile and a key split; DM0 grouped-query (HD 128)
 // prefix and suffix (the ViT attention, HD 64, is launch_flash_attention)
 enum AttnVariant { ATTN_PREFIX = 0, ATTN_SUFFIX = 1, ATTN_GQA128_PREFIX, ATTN_GQA128_SUFFIX };
-int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s);
+int launch_mqa_attention(const AttnP& p, int variant, hipStream_t s, int* kernels_launched = nullptr);
 // long sequences on both sides (csrc/flash.hip): 128 query rows per workgroup, K / V^T tiles shared through LDS; hd = 64
 int launch_flash_attention(const AttnP& p, int hd, hipStream_t s);
 // SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major

@@ -599,7 +599,10 @@ struct Sched {
         a.out = c->B("decoder_attn"); a.group = 8; a.out_tiled = 1; a.out_cols32 = 64; a.rows = 8 * S_d; a.keys = S_e + S_d; a.scale = 0.0625f;
         a.prefix_alloc = S_e; a.valid_len = valid_len(); a.state_rows = pi05 ? 0 : 8;
         a.nsplit = std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
-        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_SUFFIX, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
+        // the attention launch streams no weights and leaves a quarter of the CUs idle: 64 workgroups riding along it pull the 64 tiles
+        // (64 KB each) of the output projection that follows towards the caches (measured: 0.7 us per layer)
+        a.pf_attn = PrefetchP{{(const char*)c->TW("t_decoder_attn_o_w", i)}, {65536}, {64}};
+        if (c->want("suffix attn")) { int nk = 1; const int rc = launch_mqa_attention(a, ATTN_SUFFIX, s, &nk); c->note(rc, "suffix attn", nk); }
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024; o.gate = pi05 ? st_attn + 2048 : nullptr;
         skinny(c->B("decoder_attn"), 2048, S_d, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
         SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 4096;
@@ -745,9 +748,10 @@ struct Sched {
         a.q = c->B("decoder_Q"); a.k = dK(i); a.vt = dVt(i); a.ldvt = kp;
         a.batch = 8; a.q_bstride = (size_t)128 * 128; a.k_bstride = (size_t)kp * 128; a.vt_bstride = (size_t)128 * kp;
         a.group = 2; a.rows = 2 * ch; a.keys = P + ch; a.scale = 0.08838834764831845f; a.prefix_alloc = P + ch;
+        a.pf_attn = PrefetchP{{(const char*)c->TW("t_decoder_attn_o_w", i)}, {65536}, {64}};      // as in suffix_layer
         a.out = c->B("decoder_attn"); a.out_tiled = 1; a.out_bcol = 256; a.out_cols32 = 64;
         a.nsplit = std::min(16, (a.keys + 127) / 128); a.partial = c->B<float>("attn_partial"); a.partial_floats = ATTN_PARTIAL_FLOATS;
-        if (c->want("suffix attn")) c->note(launch_mqa_attention(a, ATTN_GQA128_SUFFIX, s), "suffix attn", a.nsplit > 1 ? 2 : 1);
+        if (c->want("suffix attn")) { int nk = 1; const int rc = launch_mqa_attention(a, ATTN_GQA128_SUFFIX, s, &nk); c->note(rc, "suffix attn", nk); }
         SkinnyP o = tiled_io(); o.out = c->B("decoder_x"); o.ldo = 1024;
         skinny(c->B("decoder_attn"), 2048, ch, c->TW("t_decoder_attn_o_w", i), nullptr, 2048, 1024, SN_NONE, nullptr, SK_RES, o, "suffix o");
         SkinnyP g = tiled_io(); g.out = c->B("decoder_hidden"); g.ldo = 2048; g.factor_f32 = 1;
