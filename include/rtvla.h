@@ -217,6 +217,33 @@ int rtvla_linear_tile_shape(int tile, int* rows, int* cols);
 int rtvla_time_linear(const void* x, int M, int K, const void* w, int N, void* out, void* workspace, size_t workspace_bytes,
                       int tile, int nsplit, int iters, void* hip_stream, float* mean_ms);
 
+/* rtvla_attention: one attention kernel family on caller tensors, all bf16 row-major (stands where the reference calls
+ * torch SDPA, pi0_infer.py:588-596, :819-824, or its own logits / softmax / P V kernels, pi0_infer.py:1041-1120,
+ * pi05_infer.py:282-309, :382-416, dm0_infer.py:822-826, :913-918):
+ *     q   [tokens][kv_heads][group][head_dim]      k, v   [keys][kv_heads][head_dim]      out   as q
+ * out = softmax(mask(scale q k^T)) v per K/V head, each shared by `group` query heads.  `kind` fixes the kernel and with it
+ * head_dim and group:
+ *     RTVLA_ATTN_GEMMA_PREFIX  (256, 8)  the Gemma-2B prefix pass            RTVLA_ATTN_GEMMA_SUFFIX  (256, 8)  the action-expert pass
+ *     RTVLA_ATTN_GQA128_PREFIX (128, 2)  DM0 prefix, causal                  RTVLA_ATTN_GQA128_SUFFIX (128, 2)  DM0 action expert
+ *     RTVLA_ATTN_VIT64         (64, 1)   DM0 ViT (keys == tokens)            RTVLA_ATTN_SIGLIP        (72, 1)   SigLIP: tokens == keys == 256 x
+ *                                                                                                                 views, kv_heads == 16, every view apart
+ * Mask (the reference's predicate, pi0_infer.py:1089-1096, pi05_infer.py:294-299): key j is visible to query token t iff
+ *     j < prefix_alloc ? j < valid_len : (t >= state_tokens || j == prefix_alloc)
+ * and, for the causal kind, j <= t.  valid_len is read from device memory (`valid_len_dev`, int32) or is prefix_alloc when
+ * that pointer is null; prefix_alloc = keys means no suffix part.  The two suffix kinds split the keys over workgroups and
+ * combine fp32 partials in a second launch, as in the forward.  `workspace`: rtvla_attention_workspace_bytes, 256-byte
+ * aligned (operands re-laid out in the kernels' fragment order, partial records).  RTVLA_ERR_LIMIT for shapes outside a
+ * kind's range (suffix kinds: at most 128 tokens; the vision kinds take no mask; the SigLIP kernel has scale = 72^-1/2 built in
+ * and refuses another). */
+enum rtvla_attention_kind {
+    RTVLA_ATTN_GEMMA_PREFIX = 0, RTVLA_ATTN_GEMMA_SUFFIX = 1, RTVLA_ATTN_GQA128_PREFIX = 2, RTVLA_ATTN_GQA128_SUFFIX = 3,
+    RTVLA_ATTN_VIT64 = 4, RTVLA_ATTN_SIGLIP = 5
+};
+size_t rtvla_attention_workspace_bytes(int kind, int tokens, int keys, int kv_heads);
+int rtvla_attention(int kind, const void* q, const void* k, const void* v, void* out, int tokens, int keys, int kv_heads,
+                    float scale, int prefix_alloc, const int32_t* valid_len_dev, int state_tokens, void* workspace,
+                    size_t workspace_bytes, void* hip_stream);
+
 /* ---- observation pre-/post-processing either side of the forward (context-free, capturable) ----------------
  * The reference does these on the host per observation (test.py:88-201).  All pointers are device pointers. */
 

@@ -559,7 +559,42 @@ int launch_mqa_inst(AttnP p, hipStream_t s, int* nk) {
     return hipGetLastError() == hipSuccess ? 0 : 5;
 }
 
+// unit-level entry point only: caller tensors -> operand layouts
+__global__ void attn_tile_operands_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v, bf16_t* __restrict__ qt,
+                                          bf16_t* __restrict__ kt, bf16_t* __restrict__ vtt, int tokens, int keys, int kv_heads, int group, int hd, int hd_pad,
+                                          size_t q_bstride, size_t k_bstride, size_t vt_bstride, int keys_pad, int seq) {
+    const size_t nq = (size_t)tokens * kv_heads * group * hd, nk = (size_t)keys * kv_heads * hd;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nq) {
+        const int d = (int)(i % hd); size_t t = i / hd;
+        const int h = (int)(t % group); t /= group;
+        const int b = (int)(t % kv_heads); int tok = (int)(t / kv_heads);
+        int bb = b;
+        if (seq > 0) { bb = (tok / seq) * kv_heads + b; tok %= seq; }
+        qt[(size_t)bb * q_bstride + ft_index(tok * group + h, d, hd_pad >> 5)] = q[i];
+        return;
+    }
+    i -= nq;
+    if (i >= 2 * nk) return;
+    const bool is_v = i >= nk;
+    if (is_v) i -= nk;
+    const int d = (int)(i % hd); size_t t = i / hd;
+    const int b = (int)(t % kv_heads); int key = (int)(t / kv_heads);
+    int bb = b;
+    if (seq > 0) { bb = (key / seq) * kv_heads + b; key %= seq; }
+    if (is_v) vtt[(size_t)bb * vt_bstride + vt_index(d, key, keys_pad >> 5)] = v[i];
+    else kt[(size_t)bb * k_bstride + ft_index(key, d, hd_pad >> 5)] = k[i];
+}
+
 }  // namespace
+
+void launch_attn_tile_operands(const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* qt, bf16_t* kt, bf16_t* vtt, int tokens, int keys,
+                               int kv_heads, int group, int hd, int hd_pad, size_t q_bstride, size_t k_bstride, size_t vt_bstride, int keys_pad,
+                               int seq, hipStream_t s) {
+    const size_t n = (size_t)tokens * kv_heads * group * hd + 2 * (size_t)keys * kv_heads * hd;
+    hipLaunchKernelGGL(attn_tile_operands_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, q, k, v, qt, kt, vtt, tokens, keys, kv_heads, group, hd,
+                       hd_pad, q_bstride, k_bstride, vt_bstride, keys_pad, seq);
+}
 
 int launch_mqa_attention(const AttnP& p0, int variant, hipStream_t s, int* nk) {
     AttnP p = p0;

@@ -168,6 +168,14 @@ int launch_flash_attention(const AttnP& p, int hd, hipStream_t s);
 // SigLIP attention: q, k fragment-tiled [views*16][256][96], vt tiled [views*16][80][256], out row-major
 void launch_vision_attention(const bf16_t* q, const bf16_t* k, const bf16_t* vt, bf16_t* out, int views, hipStream_t s);
 
+// Row-major q [tokens][kv_heads][group][hd], k / v [keys][kv_heads][hd] -> the kernels' layouts per K/V head b: Q fragment-tiled
+// [row = local token * group + head][hd_pad] at qt + b' * q_bstride, K fragment-tiled [key][hd_pad], V^T tiled [hd][keys_pad];
+// with seq > 0 the tokens / keys form independent sequences of `seq` (SigLIP views) and b' = sequence * kv_heads + b.  The
+// destination must be zero beforehand (padding).
+void launch_attn_tile_operands(const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* qt, bf16_t* kt, bf16_t* vtt, int tokens, int keys,
+                               int kv_heads, int group, int hd, int hd_pad, size_t q_bstride, size_t k_bstride, size_t vt_bstride, int keys_pad,
+                               int seq, hipStream_t s);
+
 // ----- small helpers ------------------------------------------------------------------------
 void launch_prompt_stage(const bf16_t* emb, int vocab, const int* ids, const int* valid_len, bf16_t* x_rows, int prompt_rows, int s_v,
                          float scale, const bf16_t* rope_full, int rope_rows, bf16_t* dec_rope, int dec_rows, hipStream_t s);

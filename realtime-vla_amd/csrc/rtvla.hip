@@ -6,6 +6,7 @@
 #include "kernels.h"
 #include "tuning.h"
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -1333,6 +1334,90 @@ int rtvla_linear_tile_shape(int tile, int* rows, int* cols) {
     if (tile < 0 || tile >= (int)TILE_COUNT || !rows || !cols) return RTVLA_ERR_ARG;
     *rows = gemm_tile_bm(tile); *cols = gemm_tile_bn(tile);
     return RTVLA_OK;
+}
+
+// ---- unit-level attention on caller tensors (per-kernel parity tests) ----
+namespace {
+struct AttnPlan { int hd, hd_pad, vd_pad, group, rows_pad, keys_pad, batch, nsplit; size_t q_off, k_off, vt_off, part_off, part_floats, total; };
+
+int plan_attention(int kind, int tokens, int keys, int kv_heads, AttnPlan* out) {
+    if (tokens <= 0 || keys <= 0 || kv_heads <= 0) return RTVLA_ERR_ARG;
+    AttnPlan p{};
+    p.batch = kv_heads; p.nsplit = 1;
+    int seq_rows = tokens, seq_keys = keys;
+    switch (kind) {
+        case RTVLA_ATTN_GEMMA_PREFIX: case RTVLA_ATTN_GEMMA_SUFFIX: p.hd = p.hd_pad = p.vd_pad = 256; p.group = 8; if (kv_heads != 1) return RTVLA_ERR_LIMIT; break;
+        case RTVLA_ATTN_GQA128_PREFIX: case RTVLA_ATTN_GQA128_SUFFIX: p.hd = p.hd_pad = p.vd_pad = 128; p.group = 2; break;
+        case RTVLA_ATTN_VIT64: p.hd = p.hd_pad = p.vd_pad = 64; p.group = 1; if (keys != tokens) return RTVLA_ERR_LIMIT; break;
+        case RTVLA_ATTN_SIGLIP:
+            p.hd = 72; p.hd_pad = 96; p.vd_pad = 80; p.group = 1;
+            if (kv_heads != 16 || keys != tokens || tokens % 256 || tokens > 4 * 256) return RTVLA_ERR_LIMIT;
+            p.batch = 16 * (tokens / 256); seq_rows = seq_keys = 256;
+            break;
+        default: return RTVLA_ERR_ARG;
+    }
+    if (tokens > 16384 || keys > 16384 || kv_heads > 64) return RTVLA_ERR_LIMIT;
+    const bool suffix = kind == RTVLA_ATTN_GEMMA_SUFFIX || kind == RTVLA_ATTN_GQA128_SUFFIX;
+    if (suffix && tokens > 128) return RTVLA_ERR_LIMIT;                       // the action-expert passes hold at most 128 rows per head
+    p.rows_pad = ((seq_rows * p.group + 127) / 128) * 128;
+    p.keys_pad = ((seq_keys + 63) / 64) * 64;
+    if (suffix) p.nsplit = std::min(16, (keys + 127) / 128);                 // as Sched::suffix_layer
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    p.q_off = 0;
+    p.k_off = up((size_t)p.batch * p.rows_pad * p.hd_pad * 2);
+    p.vt_off = p.k_off + up((size_t)p.batch * p.keys_pad * p.hd_pad * 2);
+    p.part_off = p.vt_off + up((size_t)p.batch * p.vd_pad * p.keys_pad * 2);
+    p.part_floats = p.nsplit > 1 ? (size_t)p.batch * ((seq_rows * p.group + 15) / 16) * p.nsplit * ((p.hd / 16) * 256 + 32) : 0;
+    p.total = p.part_off + up(p.part_floats * 4);
+    *out = p;
+    return RTVLA_OK;
+}
+}  // namespace
+
+size_t rtvla_attention_workspace_bytes(int kind, int tokens, int keys, int kv_heads) {
+    AttnPlan pl;
+    return plan_attention(kind, tokens, keys, kv_heads, &pl) == RTVLA_OK ? pl.total : 0;
+}
+
+int rtvla_attention(int kind, const void* q, const void* k, const void* v, void* out, int tokens, int keys, int kv_heads, float scale, int prefix_alloc,
+                    const int32_t* valid_len_dev, int state_tokens, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !k || !v || !out || !workspace || ((uintptr_t)workspace & 255)) return RTVLA_ERR_ARG;
+    AttnPlan pl;
+    if (int rc = plan_attention(kind, tokens, keys, kv_heads, &pl)) return rc;
+    if (workspace_bytes < pl.total) return RTVLA_ERR_SIZE;
+    if (prefix_alloc < 0 || prefix_alloc > keys || state_tokens < 0 || state_tokens > tokens) return RTVLA_ERR_ARG;
+    const bool masked = prefix_alloc < keys || valid_len_dev || state_tokens;
+    if (masked && (kind == RTVLA_ATTN_VIT64 || kind == RTVLA_ATTN_SIGLIP)) return RTVLA_ERR_LIMIT;      // the vision kernels take no masks
+    if (kind == RTVLA_ATTN_SIGLIP && fabsf(scale - 0.11785113019775792f) > 1e-6f) return RTVLA_ERR_LIMIT;   // 72^-1/2 is built into that kernel
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    bf16_t* qt = (bf16_t*)(ws + pl.q_off); bf16_t* kt = (bf16_t*)(ws + pl.k_off); bf16_t* vtt = (bf16_t*)(ws + pl.vt_off);
+    launch_fill_zero(ws, pl.part_off, s);
+    const size_t qb = (size_t)pl.rows_pad * pl.hd_pad, kb = (size_t)pl.keys_pad * pl.hd_pad, vb = (size_t)pl.vd_pad * pl.keys_pad;
+    launch_attn_tile_operands((const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, qt, kt, vtt, tokens, keys, kv_heads, pl.group, pl.hd, pl.hd_pad, qb, kb, vb,
+                              pl.keys_pad, kind == RTVLA_ATTN_SIGLIP ? 256 : 0, s);
+    int rc = 0;
+    if (kind == RTVLA_ATTN_SIGLIP) {
+        launch_vision_attention(qt, kt, vtt, (bf16_t*)out, tokens / 256, s);
+    } else {
+        AttnP a{};
+        a.q = qt; a.k = kt; a.vt = vtt; a.ldvt = pl.keys_pad;
+        a.batch = kv_heads; a.q_bstride = qb; a.k_bstride = kb; a.vt_bstride = vb;
+        a.group = pl.group; a.rows = pl.group * tokens; a.keys = keys; a.scale = scale;
+        a.out = (bf16_t*)out; a.ld_tok = kv_heads * pl.group * pl.hd; a.batch_inner = kv_heads; a.out_istride = (size_t)pl.group * pl.hd;
+        a.prefix_alloc = prefix_alloc; a.valid_len = valid_len_dev; a.state_rows = state_tokens * pl.group;
+        a.causal = kind == RTVLA_ATTN_GQA128_PREFIX;
+        a.nsplit = pl.nsplit; a.partial = (float*)(ws + pl.part_off); a.partial_floats = pl.part_floats;
+        switch (kind) {
+            case RTVLA_ATTN_GEMMA_PREFIX:  rc = launch_mqa_attention(a, ATTN_PREFIX, s); break;
+            case RTVLA_ATTN_GEMMA_SUFFIX:  rc = launch_mqa_attention(a, ATTN_SUFFIX, s); break;
+            case RTVLA_ATTN_GQA128_PREFIX: rc = launch_mqa_attention(a, ATTN_GQA128_PREFIX, s); break;
+            case RTVLA_ATTN_GQA128_SUFFIX: rc = launch_mqa_attention(a, ATTN_GQA128_SUFFIX, s); break;
+            case RTVLA_ATTN_VIT64:         rc = launch_flash_attention(a, 64, s); break;
+        }
+    }
+    if (rc) return rc == 3 ? RTVLA_ERR_LIMIT : RTVLA_ERR_DEVICE;
+    return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
 }
 
 size_t rtvla_pretile_elems(int K, int N) { return (K > 0 && N > 0) ? tiled_elems(K, N) : 0; }

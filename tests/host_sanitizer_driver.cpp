@@ -135,6 +135,23 @@ int main() {
     CHECK(rtvla_linear_tile_shape(0, nullptr, nullptr) == RTVLA_ERR_ARG);
     CHECK(rtvla_pretile_elems(588, 1152) == (size_t)72 * 20 * 512 && rtvla_pretile_elems(0, 16) == 0 && rtvla_pretile_elems(16, -1) == 0);
     CHECK(rtvla_pretile(nullptr, 16, 16, p, nullptr) == RTVLA_ERR_ARG);
+    // ---- unit-level attention: planning and argument checks ----
+    for (int kind = -1; kind <= 6; ++kind)
+        for (int tokens : {0, 1, 51, 128, 129, 256, 768, 2705, 20000})
+            for (int keys : {0, 1, 33, 256, 768, 839, 2277, 2705})
+                for (int heads : {0, 1, 8, 16, 65}) {
+                    const size_t b = rtvla_attention_workspace_bytes(kind, tokens, keys, heads);
+                    if (kind < 0 || kind > 5 || tokens <= 0 || keys <= 0 || heads <= 0 || heads > 64 || tokens > 16384) CHECK(b == 0);
+                    if (b) CHECK(b >= (size_t)keys * heads * 64 * 2 && b < ((size_t)8 << 30));
+                }
+    CHECK(rtvla_attention_workspace_bytes(RTVLA_ATTN_GEMMA_SUFFIX, 129, 900, 1) == 0);
+    CHECK(rtvla_attention_workspace_bytes(RTVLA_ATTN_GEMMA_PREFIX, 788, 788, 2) == 0);
+    CHECK(rtvla_attention_workspace_bytes(RTVLA_ATTN_SIGLIP, 768, 768, 16) > 0 && rtvla_attention_workspace_bytes(RTVLA_ATTN_SIGLIP, 700, 700, 16) == 0);
+    CHECK(rtvla_attention(RTVLA_ATTN_GEMMA_PREFIX, p, p, p, p, 788, 788, 1, 0.0625f, 788, nullptr, 0, p, 16, nullptr) == RTVLA_ERR_SIZE);
+    CHECK(rtvla_attention(RTVLA_ATTN_GEMMA_PREFIX, nullptr, p, p, p, 788, 788, 1, 0.0625f, 788, nullptr, 0, p, (size_t)1 << 30, nullptr) == RTVLA_ERR_ARG);
+    CHECK(rtvla_attention(RTVLA_ATTN_GEMMA_SUFFIX, p, p, p, p, 51, 839, 1, 0.0625f, 900, nullptr, 1, p, (size_t)1 << 30, nullptr) == RTVLA_ERR_ARG);
+    CHECK(rtvla_attention(RTVLA_ATTN_VIT64, p, p, p, p, 100, 100, 4, 0.125f, 50, nullptr, 0, p, (size_t)1 << 30, nullptr) == RTVLA_ERR_LIMIT);
+    CHECK(rtvla_attention(RTVLA_ATTN_SIGLIP, p, p, p, p, 256, 256, 16, 0.5f, 256, nullptr, 0, p, (size_t)1 << 30, nullptr) == RTVLA_ERR_LIMIT);
     // ---- pre-/post-processing: argument and size checks come before any launch ----
     CHECK(rtvla_preprocess_image_scratch(0, 10) == 0 && rtvla_preprocess_image_scratch(480, 640) >= (size_t)480 * 224 * 3);
     CHECK(rtvla_preprocess_image(nullptr, 480, 640, p, p, 1 << 20, nullptr) == RTVLA_ERR_ARG);

@@ -297,7 +297,11 @@ def test_pi0_full_size_headline_shape_with_random_norms():
 
 
 def test_c5_prefix_stress_sustained_replay():
-    """968-token prefix (1019 keys): 100 replays with fresh noise; every 25th checked against eager."""
+    """BASELINE configuration 5 as specified: 968-token prefix (1019 keys), a sustained loop of 1000 replays of the captured
+    graph, fresh N(0,1) noise every iteration, p50 / p99 of the wall-clock forward reported (method of
+    /root/reference/benchmark.py:17-33).  Every 100th iteration is re-run eagerly and must agree bit for bit; the
+    latency bound is loose (twice the 15 ms target of the smaller headline shape) so that a busy box cannot fail the test."""
+    import time
     from pi0_infer import Pi0Inference
     from oracle import pi0 as o0
     ck = syn.pi0_checkpoint(1234, 200, "cuda:0")
@@ -306,15 +310,26 @@ def test_c5_prefix_stress_sustained_replay():
     ref = o0.forward({k: v.cpu() for k, v in ck.items()}, img.cpu(), state.cpu(), noise.cpu())
     out = m.forward(img, state, noise).float().cpu()
     assert (out - ref).abs().mean().item() <= MAE_TOL
-    for it in range(100):
-        nz = syn.observation(1234, 3, 50, "cuda:0", draw=it)[2]
-        got = m.forward(img, state, nz).clone()
-        if it % 25 == 0:
+    times, finite = [], torch.ones((), dtype=torch.bool, device="cuda:0")
+    for it in range(1000):
+        nz = syn.normal_bf16(1234, "diffusion_noise/%d" % it, (50, 32), 1.0, "cuda:0")     # a fresh draw, made before the clock starts
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        got = m.forward(img, state, nz)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+        finite &= torch.isfinite(got.float()).all()
+        if it % 100 == 0:
+            got = got.clone()
             m.buffers["diffusion_noise"].copy_(nz)
             m.record_run()
             torch.cuda.synchronize()
-            assert torch.equal(got, m.buffers["diffusion_noise"])
-        assert torch.isfinite(got.float()).all()
+            assert torch.equal(got, m.buffers["diffusion_noise"]), "replay %d differs from the eager run" % it
+    assert bool(finite)
+    st = sorted(times)
+    p50, p99 = st[len(st) // 2], st[int(0.99 * len(st))]
+    print("\n[c5] 1000 sustained replays, fresh noise each: p50 %.3f ms, p99 %.3f ms, max %.3f ms" % (p50, p99, st[-1]))
+    assert p50 <= 30.0
     assert torch.equal(m.forward(img, state, noise).float().cpu(), out)
 
 
