@@ -9,13 +9,15 @@ from . import ops
 from .ops import f32, gemm
 
 
-def vision_layer(w, i, x, rnd):
+def vision_layer(w, i, x, rnd, taps=None):
     """pi0_infer.py:607-646, one SigLIP layer: LN -> QKV(+bias) -> attention -> O(+bias) + residual ->
-    LN -> up(+bias) -> GELU -> down(+bias) + residual."""
+    LN -> up(+bias) -> GELU -> down(+bias) + residual.  (taps: the stream between the two halves as "vision_mid/i".)"""
     n = rnd(ops.layer_norm(x, w["vision_pre_attn_norm_w"][i], w["vision_pre_attn_norm_b"][i]))
     qkv = rnd(f32(w["vision_attn_qkv_b"][i]) + gemm(n, w["vision_attn_qkv_w"][i]))
     a = ops.vision_attention(qkv, rnd)
     x = rnd(x + f32(w["vision_attn_o_b"][i]) + gemm(a, w["vision_attn_o_w"][i]))
+    if taps is not None:
+        taps["vision_mid/%d" % i] = x.clone()
     n = rnd(ops.layer_norm(x, w["vision_pre_ffn_norm_w"][i], w["vision_pre_ffn_norm_b"][i]))
     h = rnd(ops.gelu_tanh(f32(w["vision_ffn_up_b"][i]) + gemm(n, w["vision_ffn_up_w"][i])))
     return rnd(x + f32(w["vision_ffn_down_b"][i]) + gemm(h, w["vision_ffn_down_w"][i]))
@@ -29,7 +31,7 @@ def vision_encoder(w, images, rnd, taps=None):
     if taps is not None:
         taps["vision_embed"] = x.clone()
     for i in range(w["vision_attn_qkv_w"].shape[0]):
-        x = vision_layer(w, i, x, rnd)
+        x = vision_layer(w, i, x, rnd, taps)
         if taps is not None:
             taps["vision_x/%d" % i] = x.clone()
     return x
