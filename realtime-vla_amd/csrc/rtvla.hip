@@ -54,6 +54,8 @@ struct rtvla_ctx {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     hipStream_t timing_stream = nullptr;     // the measurement helpers capture graphs, which the null stream cannot
+    hipStream_t fork_stream = nullptr;       // second branch of the captured graph (default priority), see Sched::prefix_with_first_step
+    std::vector<hipEvent_t> fork_events;     // one per prefix layer + fork + join
     std::string err;
     int launches = 0;              // scheduler launches enqueued so far (index space of rtvla_time_launch)
     int kernels = 0;               // kernels behind them (the key-split attention is two)
@@ -527,10 +529,17 @@ struct Sched {
     bf16_t* Vt(int i) { return c->B("encoder_Vt") + (size_t)i * 256 * c->keys_pad; }
     const int* valid_len() { return pi05 ? (const int*)c->tensors[c->tindex.at("valid_encoder_len")].ptr : nullptr; }
 
-    void prefix_layer(int i) {
-        const int S_e = c->S_e, L = d.llm_layers;
+    void prefix_layer(int i) { prefix_layer_kv(i); prefix_layer_rest(i); }
+
+    // the part of a prefix layer that fills its K / V cache rows: all that the action expert's layer i needs of the prefix
+    void prefix_layer_kv(int i) {
+        const int S_e = c->S_e;
         GemmP e{}; e.rope = c->W("encoder_rope_weights"); e.q = c->B("encoder_Q"); e.k = Kc(i); e.vt = Vt(i); e.ldvt = c->keys_pad;
         gemm(c->B("encoder_x_norm"), XN_LD, S_e, S_e, c->TW("t_encoder_attn_qkv_w", i), nullptr, 2048, 2560, EPI_QKV_ROPE, e, "prefix qkv");
+    }
+
+    void prefix_layer_rest(int i) {
+        const int S_e = c->S_e, L = d.llm_layers;
         if (i == L - 1) return;                      // the last layer only fills the KV cache
         AttnP a{};
         a.q = c->B("encoder_Q"); a.k = Kc(i); a.vt = Vt(i); a.ldvt = c->keys_pad;
@@ -696,7 +705,9 @@ struct Sched {
     }
 
     // dm0_infer.py:874-951
-    void dm0_prefix_layer(int i) {
+    void dm0_prefix_layer(int i) { dm0_prefix_layer_kv(i); dm0_prefix_layer_rest(i); }
+
+    void dm0_prefix_layer_kv(int i) {
         const int P = c->S_e, kp = c->keys_pad;
         const size_t qstride = (size_t)((2 * P + 31) / 32) * 32 * 128;
         GemmP e{}; e.out = c->B("prefix_qkv"); e.ldo = 4096; e.bias = c->B("const_zeros");
@@ -706,6 +717,11 @@ struct Sched {
                                    c->W("prefix_rope_weights"), c->B("prefix_Q"), qstride, dK(i), (size_t)kp * 128, dVt(i), (size_t)128 * kp, kp >> 5, 0, P, s);
             c->note(0, "prefix qk-norm rope");
         }
+    }
+
+    void dm0_prefix_layer_rest(int i) {
+        const int P = c->S_e, kp = c->keys_pad;
+        const size_t qstride = (size_t)((2 * P + 31) / 32) * 32 * 128;
         if (i == d.llm_layers - 1) return;           // the action expert reads only the K / V cache of the last prefix layer
         AttnP a{};
         a.q = c->B("prefix_Q"); a.k = dK(i); a.vt = dVt(i); a.ldvt = kp;
@@ -815,12 +831,14 @@ struct Sched {
         return 0;
     }
 
-    void dm0_forward() {
+    void dm0_forward(hipStream_t fork = nullptr, hipEvent_t* ev = nullptr) {
         dm0_vision_embed();
         for (int i = 0; i < d.vision_layers; ++i) dm0_vision_layer(i);
         dm0_project();
-        for (int i = 0; i < d.llm_layers; ++i) dm0_prefix_layer(i);
-        for (int t = 0; t < d.num_steps; ++t) {
+        prefix_with_first_step(fork, ev, [&](int i) { dm0_prefix_layer_kv(i); }, [&](int i) { dm0_prefix_layer_rest(i); },
+                               [&]() { dm0_step_begin(0); }, [&](int i) { dm0_suffix_layer(0, i); });
+        dm0_step_end(0);
+        for (int t = 1; t < d.num_steps; ++t) {
             dm0_step_begin(t);
             for (int i = 0; i < d.llm_layers; ++i) dm0_suffix_layer(t, i);
             dm0_step_end(t);
@@ -845,14 +863,57 @@ struct Sched {
         return 0;
     }
 
-    void forward() {
-        if (d.model == RTVLA_DM0) { dm0_forward(); return; }
+    // Layer i of the action expert's FIRST flow step needs of the prefix pass only the K / V rows of prefix layer i, which exist as
+    // soon as that layer's QKV launch is done.  With a side stream (`fork`, only while both streams are being captured into one graph)
+    // the first flow step therefore runs as a second branch of the graph next to prefix layers i+1 ..: its small latency-bound
+    // launches fill the gaps of the large GEMMs instead of following them.  Same launches, same operands, same results as the
+    // one-stream order.  Returns a HIP error from the event calls, if any.
+    hipError_t fork_step0 = hipSuccess;
+    template <typename KV, typename Rest, typename Begin, typename Layer>
+    void prefix_with_first_step(hipStream_t fork, hipEvent_t* ev, KV kv, Rest rest, Begin begin, Layer layer) {
+        const int L = d.llm_layers;
+        if (!fork) {
+            for (int i = 0; i < L; ++i) { kv(i); rest(i); }
+            begin();
+            for (int i = 0; i < L; ++i) layer(i);
+            return;
+        }
+        hipStream_t main = s;
+        auto ok = [&](hipError_t e) { if (e != hipSuccess && fork_step0 == hipSuccess) fork_step0 = e; };
+        // An edge between the branches costs the main chain ~10 us (measured), so the first flow step follows in groups: after the
+        // K / V launch of prefix layers L-2, L-2-G, L-2-2G, ... the side branch runs all action-expert layers whose prefix rows exist
+        // by then; the group that ends at L-2 hides under prefix layer L-2, the last layer follows the join.  (Measured, Pi0 headline
+        // shape: one edge per layer 11.87 ms, G = 3: 11.79, 6: 11.81, 9: 11.82, a single group: 11.94 = no gain; DM0 23.28 -> 23.01 ms.
+        // The large GEMMs own every register of a CU, so the side branch's workgroups take turns with them rather than run beside
+        // them: what is saved is the launch latency of the small kernels, not their CU time.)
+        const int G = tuning_fork_group(4);
+        int next = 0;
+        for (int i = 0; i < L; ++i) {
+            kv(i);
+            if (i <= L - 2 && (L - 2 - i) % G == 0) {
+                ok(hipEventRecord(ev[i], main)); ok(hipStreamWaitEvent(fork, ev[i], 0));      // (the side stream joins the capture at the first of these)
+                s = fork;
+                if (next == 0) begin();
+                for (; next <= i; ++next) layer(next);
+                s = main;
+            }
+            rest(i);
+        }
+        if (next > 0) { ok(hipEventRecord(ev[L], fork)); ok(hipStreamWaitEvent(main, ev[L], 0)); }
+        else begin();
+        for (; next < L; ++next) layer(next);
+    }
+
+    void forward(hipStream_t fork = nullptr, hipEvent_t* ev = nullptr) {
+        if (d.model == RTVLA_DM0) { dm0_forward(fork, ev); return; }
         vision_embed();
         for (int i = 0; i < d.vision_layers; ++i) vision_layer(i);
         project();
-        for (int i = 0; i < d.llm_layers; ++i) prefix_layer(i);
         suffix_init();
-        for (int t = 0; t < d.num_steps; ++t) {
+        prefix_with_first_step(fork, ev, [&](int i) { prefix_layer_kv(i); }, [&](int i) { prefix_layer_rest(i); },
+                               [&]() { suffix_step_begin(0); }, [&](int i) { suffix_layer(0, i); });
+        suffix_step_end(0);
+        for (int t = 1; t < d.num_steps; ++t) {
             suffix_step_begin(t);
             for (int i = 0; i < d.llm_layers; ++i) suffix_layer(t, i);
             suffix_step_end(t);
@@ -994,6 +1055,8 @@ int rtvla_destroy(rtvla_ctx* c) {
     if (!c) return RTVLA_ERR_ARG;
     drop_graph(c);
     if (c->timing_stream) hipStreamDestroy(c->timing_stream);
+    if (c->fork_stream) hipStreamDestroy(c->fork_stream);
+    for (hipEvent_t e : c->fork_events) hipEventDestroy(e);
     delete c;
     return RTVLA_OK;
 }
@@ -1095,12 +1158,21 @@ int rtvla_graph_capture(rtvla_ctx* c, void* stream) {
     hipError_t e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(c, e, "eager forward before capture");
     drop_graph(c);
+    // the side stream and the events that fork / join the second branch (created once, outside the capture)
+    if (!c->fork_stream && hipStreamCreateWithFlags(&c->fork_stream, hipStreamNonBlocking) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "side stream");
+    while ((int)c->fork_events.size() < c->d.llm_layers + 2) {
+        hipEvent_t ev = nullptr;
+        if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) return c->fail(RTVLA_ERR_DEVICE, "hipEventCreate");
+        c->fork_events.push_back(ev);
+    }
     e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) return hip_fail(c, e, "hipStreamBeginCapture");
     c->status = 0; c->launches = 0; c->kernels = 0;
-    Sched(c, s).forward();
+    Sched sc(c, s);
+    sc.forward(c->fork_stream, c->fork_events.data());
     e = hipStreamEndCapture(s, &c->graph);
     if (e != hipSuccess) return hip_fail(c, e, "hipStreamEndCapture");
+    if (sc.fork_step0 != hipSuccess) return hip_fail(c, sc.fork_step0, "forking the first flow step");
     if (c->status) return c->status;
     e = hipGraphInstantiate(&c->exec, c->graph, nullptr, nullptr, 0);
     if (e != hipSuccess) return hip_fail(c, e, "hipGraphInstantiate");

@@ -2,6 +2,7 @@
 // RTVLA_TUNING: both hooks are then empty inline functions and the library reads no environment variable.  A variant build
 // (build.py -DRTVLA_TUNING -o other.so) lets a sweep force the block tile and split-K factor the cost model would pick:
 //   RTVLA_FORCE_TILE=<GemmTile>  RTVLA_FORCE_SPLIT=<n>  RTVLA_FORCE_FOR=<substring of the launch name>  RTVLA_PRINT_TILES=1
+// and set how many action-expert layers of the first flow step follow the prefix pass per graph-branch edge: RTVLA_FORK_GROUP=<n>
 #pragma once
 #ifdef RTVLA_TUNING
 #include <cstdio>
@@ -19,7 +20,9 @@ inline void tuning_report_tile(const char* what, int M, int N, int stages, int b
     if (getenv("RTVLA_PRINT_TILES"))
         fprintf(stderr, "rtvla tile choice: %-18s M=%d N=%d stages=%d -> %dx%d split %d (model %.1f us)\n", what, M, N, stages, bm, bn, nsplit, model_us);
 }
+inline int tuning_fork_group(int dflt) { const char* e = getenv("RTVLA_FORK_GROUP"); return e && atoi(e) > 0 ? atoi(e) : dflt; }
 #else
+inline int tuning_fork_group(int dflt) { return dflt; }
 inline bool tuning_forced_tile(const char*, bool, int*, int*) { return false; }
 inline void tuning_report_tile(const char*, int, int, int, int, int, int, double) {}
 #endif

@@ -220,6 +220,10 @@ def check_case(case, gold_key=None, gold_file="golden_small.pt"):
     tight = max(drift, key=lambda k: drift[k] / bound[k])
     print("\n[%s] free-running: action MAE %.5f, largest cumulative rel-L2 %.4f at %s (oracle bf16 vs fp32 there: %.4f); "
           "closest to its bound: %s at %.2f of it" % (gold_key, mae, drift[worst], worst, case.oracle_drift[worst], tight, drift[tight] / bound[tight]))
+    if os.environ.get("RTVLA_PRINT_DRIFT"):            # the whole table (pytest -s), e.g. for profiles/free_running_drift_*.md
+        print("| tap | HIP vs bf16-boundary oracle, rel-L2 | oracle bf16 vs fp32, rel-L2 | bound |\n|---|---|---|---|")
+        for k in drift:
+            print("| %s | %.5f | %.5f | %.5f |" % (k, drift[k], case.oracle_drift[k], bound[k]))
     assert torch.isfinite(staged).all()
     assert mae <= MAE_TOL
     assert drift[tight] <= bound[tight], (tight, drift[tight], bound[tight])
