@@ -134,7 +134,7 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
     static const Measured measured[] = {
         {72, 68, 1, 1, 512, TILE_64x128, 4},
         {72, 68, 1, 513, 768, TILE_128x128, 4},
-        {160, 32, 0, 769, 832, TILE_96x128, 1},
+        {160, 32, 0, 769, 1024, TILE_96x128, 1},
     };
     if (!dual)
         for (const Measured& e : measured)
