@@ -103,12 +103,13 @@ RTVLA_DEVICE float wave_sum(float v) {
 
 // Pulling weight tiles that a LATER launch of the same graph will stream towards the caches: every thread reads one word of
 // each 128-byte line of its share of a tile and throws it away (the empty asm keeps the loads alive and makes the wave wait for
-// them before it ends).  The lines land in the memory-side cache and in the L2 of the XCD the workgroup runs on, so the
-// callers give workgroup e the tile that the consuming launch will process on the same XCD (tile index = workgroup index
-// modulo 8 when both grids are dealt round-robin over the XCDs).  A launch cannot end before its riders' loads have come
-// back, and such touches draw only ~3.5 TB/s from HBM: measured on the action expert, riders that fetch the 4 MB of the
-// output projection during the suffix attention pay (0.7 us per layer), riders that fetch the 16.8 MB of the gate / up weights
-// during the attention or the merge launch lengthen that launch by 4-6 us and save 2.3 us in the consumer.
+// them before it ends).  What the later launch gains is the memory-side cache: its own L2 fills for those tiles stay the same
+// (FETCH_SIZE of the consumer does not drop: an XCD's L2 does not carry lines across a launch boundary), they only come
+// back sooner.  Workgroup e is still given the tile that the consumer processes on the same XCD (tile index = workgroup index
+// modulo 8 when both grids are dealt round-robin over the XCDs), which costs nothing.  A launch cannot end before its riders'
+// loads have come back, and such touches draw only ~3.5 TB/s from HBM: measured on the action expert, riders that fetch the
+// 4 MB of the output projection during the suffix attention pay (0.7 us per layer), riders that fetch the 16.8 MB of the gate /
+// up weights during the attention or the merge launch lengthen that launch by 4-6 us and save 2.3 us in the consumer.
 struct PrefetchP {
     const char* base[4];        // up to four weight blocks
     int tile_bytes[4];          // contiguous bytes per tile (at most 4 x 128 x the workgroup's thread count)
