@@ -217,6 +217,26 @@ int rtvla_linear_tile_shape(int tile, int* rows, int* cols);
 int rtvla_time_linear(const void* x, int M, int K, const void* w, int N, void* out, void* workspace, size_t workspace_bytes,
                       int tile, int nsplit, int iters, void* hip_stream, float* mean_ms);
 
+/* rtvla_linear_act: the fused epilogues of the large-M GEMM that write a plain row-major output (pi0_infer.py:534-561 bias + GELU,
+ * :664-691 / :727-733 GeGLU; dm0_infer.py:281-307 SwiGLU): out[M][N] =
+ *     act = RTVLA_ACT_BIAS_GELU : gelu_tanh(x w + bias)            (w_up null)
+ *     act = RTVLA_ACT_GEGLU     : gelu_tanh(x w) * (x w_up)
+ *     act = RTVLA_ACT_SWIGLU    : silu(x w) * (x w_up)
+ * Operands as for rtvla_linear; `tile` -1 (the forward's choice) or a block tile, which for the two gated forms must be 256 columns wide
+ * (RTVLA_ERR_LIMIT otherwise).
+ *
+ * rtvla_reduce_norm: the pass that follows a split-K residual GEMM (pi0_infer.py:292-346 merge_split_k_bias_res, :366-382
+ * LayerNorm, :648-663 RMSNorm): x_out[M][N] = sum of the nsplit fp32 partials [split][M][N] (nsplit 0..4, 6, 8) + bias + residual, all optional
+ * but one; xn_out = its LayerNorm with norm_w / norm_b (norm = RTVLA_NORM_LAYER) or x_out * rsqrt(mean x^2 + eps) (RTVLA_NORM_RMS),
+ * computed from the bf16-rounded x_out as the forward does; N a multiple of 4, at most 2048; x_out or xn_out may be null. */
+enum rtvla_act { RTVLA_ACT_BIAS_GELU = 1, RTVLA_ACT_GEGLU = 2, RTVLA_ACT_SWIGLU = 3 };
+enum rtvla_norm { RTVLA_NORM_NONE = 0, RTVLA_NORM_RMS = 1, RTVLA_NORM_LAYER = 2 };
+size_t rtvla_linear_act_workspace_bytes(int M, int K, int N, int act, int tile);
+int rtvla_linear_act(const void* x, int M, int K, const void* w, const void* w_up, int N, const void* bias, int act, void* out,
+                     void* workspace, size_t workspace_bytes, int tile, void* hip_stream);
+int rtvla_reduce_norm(const float* partials, int nsplit, int M, int N, const void* bias, const void* residual, int norm,
+                      const void* norm_w, const void* norm_b, float eps, void* x_out, void* xn_out, void* hip_stream);
+
 /* rtvla_attention: one attention kernel family on caller tensors, all bf16 row-major (stands where the reference calls
  * torch SDPA, pi0_infer.py:588-596, :819-824, or its own logits / softmax / P V kernels, pi0_infer.py:1041-1120,
  * pi05_infer.py:282-309, :382-416, dm0_infer.py:822-826, :913-918):

@@ -156,6 +156,13 @@ void launch_dm0_qknorm_rope(const bf16_t* qkv, int ld, const float* factor, cons
                        vt, vt_bstride, keys32, key_row0, rows);
 }
 
+__global__ void fill_f32_kernel(float* p, size_t n, float v) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+void launch_fill_f32(float* p, size_t n, float v, hipStream_t s) {
+    if (n) hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
+}
 void launch_fill_bf16(bf16_t* p, size_t n, float v, hipStream_t s) {
     if (n) hipLaunchKernelGGL(fill_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
 }

@@ -183,6 +183,7 @@ void launch_im2col(const bf16_t* images, bf16_t* patches, int ldp, int views, hi
 void launch_copy_rows(const bf16_t* src, int lds, bf16_t* dst, int ldd, int rows, int cols, hipStream_t s);
 void launch_fill_zero(void* p, size_t bytes, hipStream_t s);
 void launch_fill_bf16(bf16_t* p, size_t n, float v, hipStream_t s);
+void launch_fill_f32(float* p, size_t n, float v, hipStream_t s);
 
 // ----- DM0 (csrc/dm0.hip) ---------------------------------------------------------------------
 void launch_dm0_im2col_nchw(const bf16_t* images, bf16_t* patches, int ldp, int n_images, hipStream_t s);

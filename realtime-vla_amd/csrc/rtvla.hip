@@ -1408,6 +1408,89 @@ int rtvla_linear_tile_shape(int tile, int* rows, int* cols) {
     return RTVLA_OK;
 }
 
+// ---- unit-level fused GEMM epilogues and the reduce / normalise pass (per-kernel parity tests) ----
+namespace {
+struct ActPlan { size_t a_off, w0_off, w1_off, bias_off, scale_off, total; int K128, tile; bool dual; };
+
+int plan_linear_act(int M, int K, int N, int act, int tile, ActPlan* out) {
+    if (M <= 0 || K <= 0 || N <= 0 || (K & 7) || (N & 15)) return RTVLA_ERR_ARG;
+    if (act != RTVLA_ACT_BIAS_GELU && act != RTVLA_ACT_GEGLU && act != RTVLA_ACT_SWIGLU) return RTVLA_ERR_ARG;
+    if (tile < -1 || tile >= (int)TILE_COUNT) return RTVLA_ERR_ARG;
+    ActPlan p{};
+    p.dual = act != RTVLA_ACT_BIAS_GELU;
+    p.K128 = k32_padded(K) * 32;
+    p.tile = tile >= 0 ? tile : choose_tile(M, n16_tiles(N), k32_padded(K) / 2, p.dual, false, "linear act", p.dual ? 0 : 1).tile;
+    if (p.dual && (gemm_tile_bn(p.tile) != 256 || gemm_tile_eight_waves(p.tile))) return RTVLA_ERR_LIMIT;      // gate and up share a 256-column workgroup tile
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const int G = p.dual ? 4 : 8;
+    p.a_off = 0;
+    p.w0_off = up((size_t)M * p.K128 * 2);
+    p.w1_off = p.w0_off + up(tiled_elems_wide(K, N, G) * 2);
+    p.bias_off = p.w1_off + (p.dual ? up(tiled_elems_wide(K, N, G) * 2) : 0);
+    p.scale_off = p.bias_off + up((size_t)N * 2);
+    p.total = p.scale_off + up((size_t)M * 4);
+    *out = p;
+    return RTVLA_OK;
+}
+}  // namespace
+
+size_t rtvla_linear_act_workspace_bytes(int M, int K, int N, int act, int tile) {
+    ActPlan pl;
+    return plan_linear_act(M, K, N, act, tile, &pl) == RTVLA_OK ? pl.total : 0;
+}
+
+int rtvla_linear_act(const void* x, int M, int K, const void* w, const void* w_up, int N, const void* bias, int act, void* out, void* workspace,
+                     size_t workspace_bytes, int tile, void* stream) {
+    if (!x || !w || !out || !workspace || ((uintptr_t)workspace & 255)) return RTVLA_ERR_ARG;
+    ActPlan pl;
+    if (int rc = plan_linear_act(M, K, N, act, tile, &pl)) return rc;
+    if (pl.dual != (w_up != nullptr)) return RTVLA_ERR_ARG;
+    if (workspace_bytes < pl.total) return RTVLA_ERR_SIZE;
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    bf16_t* a = (bf16_t*)(ws + pl.a_off);
+    launch_fill_zero(a, ((size_t)M * pl.K128 * 2 + 255) & ~(size_t)255, s);
+    launch_copy_rows((const bf16_t*)x, K, a, pl.K128, M, K, s);
+    const int G = pl.dual ? 4 : 8;
+    launch_pretile((const bf16_t*)w, K, N, (bf16_t*)(ws + pl.w0_off), G, 1, s);
+    if (pl.dual) launch_pretile((const bf16_t*)w_up, K, N, (bf16_t*)(ws + pl.w1_off), G, 1, s);
+    bf16_t* zbias = (bf16_t*)(ws + pl.bias_off);
+    launch_fill_zero(zbias, ((size_t)N * 2 + 255) & ~(size_t)255, s);
+    GemmP p{};
+    p.A = a; p.lda = pl.K128; p.a_rows = M; p.M = M; p.B0 = (bf16_t*)(ws + pl.w0_off); p.B1 = pl.dual ? (bf16_t*)(ws + pl.w1_off) : nullptr;
+    p.bgroup = G; p.N16 = n16_tiles(N); p.K32p = k32_padded(K); p.nsplit = 1;
+    p.out = (bf16_t*)out; p.ldo = N; p.bias = bias ? (const bf16_t*)bias : zbias;
+    int epi = EPI_BIAS_GELU;
+    if (act == RTVLA_ACT_GEGLU) epi = EPI_GEGLU;
+    if (act == RTVLA_ACT_SWIGLU) {
+        epi = EPI_SWIGLU;
+        float* ones = (float*)(ws + pl.scale_off);                       // the SwiGLU epilogue multiplies by a per-row factor (DM0's RMS norm): 1 here
+        launch_fill_f32(ones, M, 1.0f, s);
+        p.rowscale = ones;
+    }
+    const int rc = launch_gemm(p, epi, pl.tile, s);
+    if (rc) return (rc == 2 || rc == 3) ? RTVLA_ERR_LIMIT : RTVLA_ERR_DEVICE;
+    return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
+}
+
+int rtvla_reduce_norm(const float* partials, int nsplit, int M, int N, const void* bias, const void* residual, int norm, const void* norm_w,
+                      const void* norm_b, float eps, void* x_out, void* xn_out, void* stream) {
+    if (M <= 0 || N <= 0 || (N & 3) || N > 2048) return RTVLA_ERR_ARG;
+    if (nsplit < 0 || nsplit > 8 || nsplit == 5 || nsplit == 7) return RTVLA_ERR_ARG;
+    if ((nsplit > 0 && !partials) || (nsplit == 0 && !residual) || (!x_out && !xn_out)) return RTVLA_ERR_ARG;
+    if (norm != RTVLA_NORM_NONE && norm != RTVLA_NORM_RMS && norm != RTVLA_NORM_LAYER) return RTVLA_ERR_ARG;
+    if (norm != RTVLA_NORM_NONE && !xn_out) return RTVLA_ERR_ARG;
+    if (norm == RTVLA_NORM_LAYER && (!norm_w || !norm_b)) return RTVLA_ERR_ARG;
+    ReduceP r{};
+    r.partial = partials; r.pstride = (size_t)M * N; r.ldp = N; r.nsplit = nsplit;
+    r.bias = (const bf16_t*)bias; r.res = (const bf16_t*)residual; r.ldr = N;
+    r.x = (bf16_t*)x_out; r.ldx = N; r.xn = (bf16_t*)xn_out; r.ldxn = N;
+    r.M = M; r.N = N; r.norm = norm == RTVLA_NORM_RMS ? NORM_RMS : norm == RTVLA_NORM_LAYER ? NORM_LAYER : NORM_NONE;
+    r.nw = (const bf16_t*)norm_w; r.nb = (const bf16_t*)norm_b; r.eps = eps;
+    if (launch_reduce(r, (hipStream_t)stream)) return RTVLA_ERR_DEVICE;
+    return hipGetLastError() == hipSuccess ? RTVLA_OK : RTVLA_ERR_DEVICE;
+}
+
 // ---- unit-level attention on caller tensors (per-kernel parity tests) ----
 namespace {
 struct AttnPlan { int hd, hd_pad, vd_pad, group, rows_pad, keys_pad, batch, nsplit; size_t q_off, k_off, vt_off, part_off, part_floats, total; };

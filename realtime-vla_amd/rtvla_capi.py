@@ -22,6 +22,8 @@ STAGE_SUFFIX_STEP_END = 7
 
 ERR_NAME, ERR_SIZE, ERR_STATE, ERR_LIMIT = 2, 3, 4, 7
 TILE_AUTO, TILE_SKINNY = -1, -2
+ACT_BIAS_GELU, ACT_GEGLU, ACT_SWIGLU = 1, 2, 3
+NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
 ATTN_GEMMA_PREFIX, ATTN_GEMMA_SUFFIX, ATTN_GQA128_PREFIX, ATTN_GQA128_SUFFIX, ATTN_VIT64, ATTN_SIGLIP = range(6)
 STATIC_SCRATCH_BYTES = 2160 * 224 * 3          # RTVLA_STATIC_SCRATCH_BYTES
 
@@ -70,6 +72,9 @@ SYMBOLS = {
     "rtvla_time_linear": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, ctypes.c_int, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
                                          ctypes.c_int, _P, ctypes.POINTER(ctypes.c_float)]),
     "rtvla_linear_tile_shape": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
+    "rtvla_linear_act_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "rtvla_linear_act": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _P, _P, ctypes.c_int, _P, ctypes.c_int, _P, _P, ctypes.c_size_t, ctypes.c_int, _P]),
+    "rtvla_reduce_norm": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P, _P, ctypes.c_int, _P, _P, ctypes.c_float, _P, _P, _P]),
     "rtvla_attention_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "rtvla_attention": (ctypes.c_int, [ctypes.c_int, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_int, _P,
                                        ctypes.c_int, _P, ctypes.c_size_t, _P]),

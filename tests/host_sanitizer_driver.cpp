@@ -135,6 +135,21 @@ int main() {
     CHECK(rtvla_linear_tile_shape(0, nullptr, nullptr) == RTVLA_ERR_ARG);
     CHECK(rtvla_pretile_elems(588, 1152) == (size_t)72 * 20 * 512 && rtvla_pretile_elems(0, 16) == 0 && rtvla_pretile_elems(16, -1) == 0);
     CHECK(rtvla_pretile(nullptr, 16, 16, p, nullptr) == RTVLA_ERR_ARG);
+    // ---- fused epilogues and the reduce pass: planning and argument checks ----
+    for (int act = 0; act <= 4; ++act)
+        for (int tile = -2; tile <= 13; ++tile)
+            for (int N : {16, 24, 272, 4304 - 4304 % 16, 16384}) {
+                const size_t b = rtvla_linear_act_workspace_bytes(788, 2048, N, act, tile);
+                if (act < 1 || act > 3 || tile < -1 || tile > 11 || (N & 15)) CHECK(b == 0);
+                if (b) CHECK(b >= (size_t)788 * 2048 * 2);
+            }
+    CHECK(rtvla_linear_act(p, 788, 2048, p, nullptr, 16384, nullptr, RTVLA_ACT_GEGLU, p, p, (size_t)1 << 32, -1, nullptr) == RTVLA_ERR_ARG);     // gated without w_up
+    CHECK(rtvla_linear_act(p, 788, 2048, p, p, 16384, nullptr, RTVLA_ACT_GEGLU, p, p, 16, -1, nullptr) == RTVLA_ERR_SIZE);
+    CHECK(rtvla_reduce_norm(nullptr, 2, 16, 64, nullptr, nullptr, 0, nullptr, nullptr, 1e-6f, p, nullptr, nullptr) == RTVLA_ERR_ARG);
+    CHECK(rtvla_reduce_norm((const float*)p, 5, 16, 64, nullptr, nullptr, 0, nullptr, nullptr, 1e-6f, p, nullptr, nullptr) == RTVLA_ERR_ARG);
+    CHECK(rtvla_reduce_norm((const float*)p, 2, 16, 4096, nullptr, nullptr, 0, nullptr, nullptr, 1e-6f, p, nullptr, nullptr) == RTVLA_ERR_ARG);
+    CHECK(rtvla_reduce_norm((const float*)p, 2, 16, 64, nullptr, nullptr, RTVLA_NORM_LAYER, nullptr, nullptr, 1e-5f, p, p, nullptr) == RTVLA_ERR_ARG);
+    CHECK(rtvla_reduce_norm((const float*)p, 2, 16, 64, nullptr, nullptr, RTVLA_NORM_RMS, nullptr, nullptr, 1e-6f, p, nullptr, nullptr) == RTVLA_ERR_ARG);
     // ---- unit-level attention: planning and argument checks ----
     for (int kind = -1; kind <= 6; ++kind)
         for (int tokens : {0, 1, 51, 128, 129, 256, 768, 2705, 20000})

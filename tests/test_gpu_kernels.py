@@ -127,3 +127,104 @@ def test_a_graph_captured_before_a_rebind_is_refused():
     m.record_infer_graph()
     b = m.forward(img, state, noise)
     assert b.data_ptr() == other.data_ptr() and torch.equal(a, b)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# fused GEMM epilogues with a row-major output, and the reduce / normalise pass, each on its own
+def _gelu_tanh(a):
+    return a * torch.sigmoid(1.5957691216057308 * a * (1.0 + 0.044715 * a * a))
+
+
+def _run_act(lib, capi, M, K, N, act, tile, seed=0):
+    g = torch.Generator(device="cuda:0").manual_seed(seed * 104729 + M + K + N + act)
+    x = torch.randn(M, K, device="cuda:0", generator=g).to(torch.bfloat16)
+    w = (torch.randn(K, N, device="cuda:0", generator=g) * 0.05).to(torch.bfloat16)
+    dual = act != capi.ACT_BIAS_GELU
+    w2 = (torch.randn(K, N, device="cuda:0", generator=g) * 0.05).to(torch.bfloat16) if dual else None
+    b = None if dual else torch.randn(N, device="cuda:0", generator=g).to(torch.bfloat16)
+    need = lib.rtvla_linear_act_workspace_bytes(M, K, N, act, tile)
+    if need == 0:
+        return None
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda:0")
+    out = torch.full((M, N), 77.0, dtype=torch.bfloat16, device="cuda:0")
+    rc = lib.rtvla_linear_act(_P(x.data_ptr()), M, K, _P(w.data_ptr()), _P(w2.data_ptr()) if dual else None, N, _P(b.data_ptr()) if b is not None else None,
+                              act, _P(out.data_ptr()), _P(ws.data_ptr()), need, tile, _P(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    if rc == capi.ERR_LIMIT:
+        return None
+    assert rc == 0, rc
+    a = x.float() @ w.float()
+    if act == capi.ACT_BIAS_GELU:
+        ref = _gelu_tanh(a + b.float())
+    elif act == capi.ACT_GEGLU:
+        ref = _gelu_tanh(a) * (x.float() @ w2.float())
+    else:
+        ref = a * torch.sigmoid(a) * (x.float() @ w2.float())
+    got = out.float()
+    rel = ((got - ref).norm() / ref.norm()).item()
+    excess = (got - ref).abs() / (ref.abs() * 2.0 ** -7 + 2e-3 * ref.pow(2).mean().sqrt())      # (the activations use the hardware exp2 / rcp)
+    return rel, excess.max().item()
+
+
+@pytest.mark.parametrize("M,K,N,act", [
+    (768, 1152, 4304, 1),       # SigLIP up-projection: bias + GELU
+    (788, 2048, 16384, 2),      # Gemma prefix gate / up: GeGLU, 25 row tiles in mixed blocks
+    (607, 2048, 6144, 3),       # DM0 prefix gate / up: SwiGLU
+    (8115, 1024, 4096, 1),      # DM0 ViT fc: bias + GELU on the eight-wave tile
+    (37, 136, 48, 1), (37, 136, 48, 2), (225, 264, 272, 3),      # ragged rows, K and columns
+])
+def test_fused_activation_epilogues_against_fp32(M, K, N, act):
+    import rtvla_capi as capi
+    lib = capi.load()
+    ran = 0
+    for tile, rows, cols in [(capi.TILE_AUTO, 0, 0)] + _tiles(lib):
+        if M > 1000 and tile != capi.TILE_AUTO and rows < 128:
+            continue                                        # (keeps the 8115-row case short)
+        res = _run_act(lib, capi, M, K, N, act, tile)
+        if res is None:
+            continue                                        # a gated epilogue needs a 256-column tile; the large tiles need an even stage count
+        ran += 1
+        assert res[0] <= REL_TOL and res[1] <= 1.01, ("tile %dx%d" % (rows, cols), res)
+    assert ran >= 3
+
+
+@pytest.mark.parametrize("M,N,nsplit,norm,has_bias,has_res", [
+    (768, 1152, 2, 2, True, True),        # SigLIP O projection: split 2 + bias + residual + LayerNorm
+    (768, 1152, 4, 2, True, True),        # SigLIP down projection
+    (768, 1152, 0, 2, False, True),       # LayerNorm of a stream alone (first layer)
+    (788, 2048, 1, 1, False, True),       # prefix O projection: one partial + residual + RMS norm
+    (788, 2048, 4, 1, False, True),       # prefix down projection
+    (968, 2048, 8, 1, False, True), (33, 2048, 6, 1, True, False), (5, 1024, 3, 0, True, True), (2705, 1024, 1, 2, True, True),
+])
+def test_reduce_bias_residual_norm_against_fp32(M, N, nsplit, norm, has_bias, has_res):
+    import rtvla_capi as capi
+    lib = capi.load()
+    g = torch.Generator(device="cuda:0").manual_seed(M * 31 + N + nsplit)
+    parts = torch.randn(max(nsplit, 1), M, N, device="cuda:0", generator=g)
+    bias = torch.randn(N, device="cuda:0", generator=g).bfloat16() if has_bias else None
+    res = (torch.randn(M, N, device="cuda:0", generator=g) * 2 + 0.5).bfloat16() if has_res else None
+    nw = (1 + 0.1 * torch.randn(N, device="cuda:0", generator=g)).bfloat16()
+    nb = (0.1 * torch.randn(N, device="cuda:0", generator=g)).bfloat16()
+    x = torch.full((M, N), 9.0, dtype=torch.bfloat16, device="cuda:0")
+    xn = torch.full((M, N), 9.0, dtype=torch.bfloat16, device="cuda:0")
+    eps = 1e-5 if norm == 2 else 1e-6
+    rc = lib.rtvla_reduce_norm(_P(parts.data_ptr()) if nsplit else None, nsplit, M, N, _P(bias.data_ptr()) if has_bias else None,
+                               _P(res.data_ptr()) if has_res else None, norm, _P(nw.data_ptr()), _P(nb.data_ptr()), ctypes.c_float(eps),
+                               _P(x.data_ptr()), _P(xn.data_ptr()) if norm else None, _P(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    want = (parts[:nsplit].sum(0) if nsplit else torch.zeros(M, N, device="cuda:0"))
+    if has_bias:
+        want = want + bias.float()
+    if has_res:
+        want = want + res.float()
+    assert ((x.float() - want).norm() / want.norm()).item() <= REL_TOL
+    assert ((x.float() - want).abs() <= want.abs() * 2.0 ** -7 + 1e-3).all()
+    if norm:
+        xb = x.float()                                      # the norm reads the rounded stream, as the forward's next GEMM input does
+        if norm == 2:
+            ref = torch.nn.functional.layer_norm(xb, (N,), nw.float(), nb.float(), eps)
+        else:
+            ref = xb * torch.rsqrt(xb.pow(2).mean(-1, keepdim=True) + eps)
+        assert ((xn.float() - ref).norm() / ref.norm()).item() <= REL_TOL
+        assert ((xn.float() - ref).abs() <= ref.abs() * 2.0 ** -7 + 2e-3).all()
