@@ -34,6 +34,8 @@ class Engine:
         if llm_layers is None:
             llm_layers = int(checkpoint["encoder_attn_qkv_w"].shape[0]) if "encoder_attn_qkv_w" in checkpoint else 18
         self.model, self.vision_layers, self.llm_layers, self.num_steps = model, vision_layers, llm_layers, num_steps
+        self.prefix_rows = num_views * 256 + prompt_len                       # rows of the prefix pass (as allocated)
+        self.suffix_rows = chunk_size + (1 if model == capi.PI0 else 0)       # Pi0: the state token precedes the action rows
         self.tile_cache = TileCache(tile_cache) if isinstance(tile_cache, (str, os.PathLike)) else tile_cache
         self.tile_cache_hit = None                                   # True / False after prepare() when a cache is in use
         self.ctx = capi.Context(model, num_views, prompt_len, chunk_size, num_steps, vision_layers, llm_layers)
@@ -100,6 +102,35 @@ class Engine:
         self.ctx.graph_capture(side.cuda_stream)
         side.synchronize()
         self.graph_launches = self.ctx.launch_count()      # kernel nodes in the captured graph
+
+    def reference_buffer(self, name):
+        """Row-major copy of an internal activation in the shape the reference keeps it in
+        (/root/reference/pi0_infer.py:1291-1317, pi05_infer.py:690-730): the MFMA kernels hold these tensors fragment-tiled,
+        so `buffers[name]` has other bytes than the reference's tensor of that name.  Pi0 / Pi05 names: encoder_K, encoder_V
+        ([layers][prefix + suffix rows][256]), encoder_Q ([prefix rows * 8][256]), vision_QKV ([views][256][3 * 1152]),
+        decoder_x, decoder_x_buf, decoder_q_buf, decoder_hidden.  Row-major buffers are returned as they are."""
+        B, L = self.buffers, self.llm_layers
+        if self.model == capi.DM0:
+            raise KeyError("reference_buffer covers the Pi0 / Pi05 buffers")
+        if name == "encoder_K":
+            kp = B["encoder_K"].numel() // (L * 256)
+            return torch.stack([untile_ft(B["encoder_K"].reshape(L, -1)[i], kp, 256) for i in range(L)])[:, : self.prefix_rows + self.suffix_rows]
+        if name == "encoder_V":
+            kp = B["encoder_Vt"].numel() // (L * 256)
+            return torch.stack([untile_vt(B["encoder_Vt"].reshape(L, -1)[i], 256, kp).t() for i in range(L)])[:, : self.prefix_rows + self.suffix_rows].contiguous()
+        if name in ("encoder_Q", "decoder_q_buf", "decoder_x", "decoder_x_buf", "decoder_hidden"):
+            t = B[name]
+            rows = {"encoder_Q": 8 * self.prefix_rows, "decoder_q_buf": 8 * self.suffix_rows, "decoder_x": self.suffix_rows,
+                    "decoder_x_buf": self.suffix_rows, "decoder_hidden": self.suffix_rows}[name]
+            cols = t.shape[1]
+            return untile_ft(t, t.numel() // cols, cols)[:rows]
+        if name == "vision_QKV":
+            v = B["vision_Q"].shape[0] // 16
+            q = torch.stack([untile_ft(x, 256, 96)[:, :72] for x in B["vision_Q"]]).view(v, 16, 256, 72)
+            k = torch.stack([untile_ft(x, 256, 96)[:, :72] for x in B["vision_K"]]).view(v, 16, 256, 72)
+            vv = torch.stack([untile_vt(x, 80, 256)[:72].t() for x in B["vision_Vt"]]).view(v, 16, 256, 72)
+            return torch.stack([q, k, vv], 1).permute(0, 3, 1, 2, 4).reshape(v, 256, 3 * 1152)
+        return B[name]
 
     def replay(self):
         self.ctx.graph_launch(torch.cuda.current_stream(self.device).cuda_stream)

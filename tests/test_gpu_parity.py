@@ -337,6 +337,40 @@ def test_c5_prefix_stress_sustained_replay():
     assert torch.equal(m.forward(img, state, noise).float().cpu(), out)
 
 
+def test_reference_buffer_gives_the_reference_layout_of_the_internal_activations():
+    """`Engine.reference_buffer` un-tiles the activations the MFMA kernels keep in fragment order into the tensors the reference
+    keeps under the same names (/root/reference/pi0_infer.py:1291-1317): shapes as there, prefix K / V equal to the oracle's,
+    vision_QKV consistent with the attention output it produced (torch SDPA over it, pi0_infer.py:588-596), and a row-major
+    buffer passed through unchanged."""
+    c = Case("pi0", 7, views=2, prompt=5, chunk=9, vision_layers=2, llm_layers=3)
+    c.forward(); torch.cuda.synchronize()
+    e = c.e
+    S_e, S_d = c.S_e, c.S_d
+    K, V = e.reference_buffer("encoder_K"), e.reference_buffer("encoder_V")
+    assert K.shape == (3, S_e + S_d, 256) and V.shape == (3, S_e + S_d, 256)
+    for i in range(3):
+        for got, name in ((K, "encoder_K/%d"), (V, "encoder_V/%d")):
+            want = c.taps[name % i][:S_e].float()
+            err = (got[i, :S_e].float().cpu() - want).norm() / want.norm()
+            assert err < 2e-2, (name % i, err.item())
+    assert e.reference_buffer("encoder_Q").shape == (S_e * 8, 256)
+    assert e.reference_buffer("decoder_x").shape == (S_d, 1024)
+    assert e.reference_buffer("decoder_x_buf").shape == (S_d, 1024)
+    assert e.reference_buffer("decoder_q_buf").shape == (S_d * 8, 256)
+    assert e.reference_buffer("decoder_hidden").shape == (S_d, 4096)
+    assert torch.equal(e.reference_buffer("decoder_x"), c.dec_x())
+    assert e.reference_buffer("encoder_x").data_ptr() == c.B["encoder_x"].data_ptr()
+    # the last vision layer's Q, K, V in the reference's packing reproduce that layer's attention output
+    c.run(c.capi.STAGE_VISION_EMBED)
+    c.run(c.capi.STAGE_VISION_LAYER, 0)
+    qkv = e.reference_buffer("vision_QKV")
+    assert qkv.shape == (2, 256, 3 * 1152)
+    t = qkv.float().view(-1, 256, 3, 16, 72).permute(0, 2, 3, 1, 4)
+    attn = torch.nn.functional.scaled_dot_product_attention(t[:, 0], t[:, 1], t[:, 2]).transpose(1, 2).reshape(2 * 256, 1152)
+    got = c.B["vision_attn"].float()
+    assert ((got - attn).norm() / attn.norm()).item() < 1e-2
+
+
 def test_zero_output_projection_returns_the_noise_bit_exactly():
     from pi0_infer import Pi0Inference
     ck = syn.pi0_checkpoint(3, 2, "cuda:0", 1, 2)
