@@ -34,13 +34,16 @@ def reference(kind, q, k, v, scale, prefix_alloc, valid_len, state_tokens):
     return torch.einsum("bgtk,kbd->tbgd", torch.softmax(logits, -1), v.float())
 
 
-def run(kind, tokens, keys, kv_heads, prefix_alloc=None, valid_len=None, state_tokens=0, seed=0, sharp=1.0):
+def run(kind, tokens, keys, kv_heads, prefix_alloc=None, valid_len=None, state_tokens=0, seed=0, sharp=1.0, ramp=0.0):
     lib = capi.load()
     D, G = KINDS[kind]
     g = torch.Generator(device="cuda:0").manual_seed(seed)
     q = (torch.randn(tokens, kv_heads, G, D, device="cuda:0", generator=g) * sharp).bfloat16()
     k = torch.randn(keys, kv_heads, D, device="cuda:0", generator=g).bfloat16()
     v = torch.randn(keys, kv_heads, D, device="cuda:0", generator=g).bfloat16()
+    if ramp:            # logits that climb with the key index: the running maximum grows all the way through the key loop
+        q = q.float(); q[..., 0] += 4.0; q = q.bfloat16()
+        k = k.float(); k[..., 0] += ramp * torch.arange(keys, device="cuda:0")[:, None] / keys; k = k.bfloat16()
     out = torch.full_like(q, 9.0)
     scale = D ** -0.5
     prefix_alloc = keys if prefix_alloc is None else prefix_alloc
@@ -113,9 +116,18 @@ def test_grouped_query_suffix_pass(tokens, prefix, heads):
     run(capi.ATTN_GQA128_SUFFIX, tokens, prefix + tokens, heads, seed=prefix)
 
 
-@pytest.mark.parametrize("tokens,heads", [(1, 16), (63, 3), (64, 8), (129, 16), (2705, 16)])
+@pytest.mark.parametrize("tokens,heads", [(1, 16), (63, 3), (64, 8), (96, 2), (128, 4), (129, 16), (192, 3), (200, 2), (257, 5), (2705, 16)])
 def test_vit_flash_attention(tokens, heads):
+    """One to 43 key tiles of 64: a single tile, an odd number of 32-key blocks (the half-filled last tile), three and more
+    tiles (the three LDS stages wrap), the DM0 shape."""
     run(capi.ATTN_VIT64, tokens, tokens, heads, seed=tokens)
+
+
+@pytest.mark.parametrize("tokens", [96, 700, 2705])
+def test_vit_flash_attention_with_a_maximum_that_keeps_growing(tokens):
+    """The ViT kernel rescales its accumulator only when a row maximum grew by 2^8 and moves the probabilities of the block in
+    flight to the new scale: logits that climb by ~90 bits over the keys take that path about a dozen times per row."""
+    run(capi.ATTN_VIT64, tokens, tokens, 3, seed=tokens + 1, ramp=128.0)
 
 
 @pytest.mark.parametrize("views", [1, 3])
