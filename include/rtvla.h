@@ -82,7 +82,7 @@ enum rtvla_stage {
 
 /* Library version (no reference counterpart): raised whenever a kernel or the schedule changes, so that a
  * measurement recorded for one version is not mistaken for the current kernels. */
-#define RTVLA_VERSION 8
+#define RTVLA_VERSION 9
 int rtvla_version(void);
 
 /* Create a context for one shape set.  Replaces the tensor allocation block of
