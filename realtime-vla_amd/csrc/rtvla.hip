@@ -129,12 +129,14 @@ TileChoice choose_tile(int M, int ncols16, int stages, bool dual, bool splittabl
     if (eight && M >= 4096 && stages <= 32 && ncols16 >= 128) return TileChoice{eight == 1 ? TILE8_256x256 : TILE8_128x256, 1};
     // shapes where timing the launch inside a layer (weights streamed from HBM) disagrees with the model below: the K = 4304
     // SigLIP down-projection gains from four K splits (more workgroups pulling the 9.9 MB of weights at once, 22.1 -> 19.3 us
-    // with the reduce pass at 768 rows, 20.4 -> 14.4 us at 256 rows), the 788-row prefix QKV from 96-row tiles (22.0 -> 20.5 us)
+    // with the reduce pass at 768 rows, 20.4 -> 14.4 us at 256 rows), the 788-row prefix QKV from 96-row tiles (22.0 -> 20.5 us), and so does
+    // the SigLIP QKV GEMM at three views (768 rows as 8 x 27 = 216 workgroups, one per CU, instead of 324 on 256 CUs: 14.8 -> 12.4 us)
     struct Measured { int ncols16, stages, splittable, m_lo, m_hi, tile, nsplit; };
     static const Measured measured[] = {
         {72, 68, 1, 1, 512, TILE_64x128, 4},
         {72, 68, 1, 513, 768, TILE_128x128, 4},
         {160, 32, 0, 769, 1024, TILE_96x128, 1},
+        {216, 18, 0, 673, 768, TILE_96x128, 1},
     };
     if (!dual)
         for (const Measured& e : measured)
