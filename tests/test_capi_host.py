@@ -29,6 +29,17 @@ def test_every_declared_symbol_is_exported(lib):
     assert lib.rtvla_version() >= 1
 
 
+def test_the_shipped_library_reads_no_environment(lib):
+    """The tuning hooks (forced tiles, graph-branch knobs) exist only in builds made with -DRTVLA_TUNING: the shipped library
+    imports no getenv and carries none of the knob names."""
+    import subprocess
+    syms = subprocess.run(["nm", "-D", "--undefined-only", capi.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    assert "getenv" not in syms
+    blob = open(capi.LIB_PATH, "rb").read()
+    for knob in (b"RTVLA_FORCE_TILE", b"RTVLA_FORK_GROUP", b"RTVLA_PRINT_TILES"):
+        assert knob not in blob
+
+
 def test_create_validates_dimensions(lib):
     for bad in [(capi.PI0, 0, 0, 50), (capi.PI0, 5, 0, 50), (capi.PI0, 1, -1, 50), (capi.PI0, 1, 0, 0), (3, 1, 0, 50), (capi.DM0, 0, 10, 50), (capi.DM0, 5, 10, 50)]:
         with pytest.raises(capi.RtvlaError):
